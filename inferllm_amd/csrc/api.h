@@ -19,6 +19,19 @@ int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* ou
 int illm_embed_scaled(const int32_t* tokens, const void* table, int table_dt, float* out,
                       int T, int E, int V, float scale, void* stream);
 
+// out[t, :] = table[tokens[t]] * scale + pairs[(prev * mul_prev + tokens[t] * mul_cur) mod buckets]
+// + places[row_pos[t]]: prev is the token above in the step if it belongs to the same slot, else
+// last_token[slot]; a row at position 0 takes pairs[buckets].  pairs, places may be null.  `remember`
+// (one row a sequence): last_token[slot] = tokens[t] as well.
+int illm_embed_pairs(const int32_t* tokens, const int32_t* row_pos, const int32_t* row_slot,
+                     const void* table, int table_dt, const void* pairs, int pairs_dt,
+                     const void* places, int places_dt, int32_t* last_token, float* out, int T, int E,
+                     int V, int buckets, int mul_prev, int mul_cur, int n_places, float scale,
+                     int remember, void* stream);
+// last_token[seq_slot[b]] = the last token of sequence b's rows (cu [n_seqs + 1] row offsets).
+int illm_remember_last(const int32_t* tokens, const int32_t* cu, const int32_t* seq_slot,
+                       int32_t* last_token, int n_seqs, void* stream);
+
 // out[i] = float32(a[i]) + float32(b[i]): the two outputs of a block whose parts read the same rows.
 int illm_sum_rows(const void* a, int a_dt, const void* b, int b_dt, float* out, size_t n,
                   void* stream);
@@ -28,6 +41,8 @@ int illm_sum_rows_scaled(const void* a, int a_dt, float sa, const void* b, int b
 
 // out[i] = max(x[i], 0)^2.
 int illm_relu_squared(const void* x, void* out, int dt, size_t n, void* stream);
+// out[i] = 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))).
+int illm_gelu_tanh(const void* x, void* out, int dt, size_t n, void* stream);
 
 // Residual add and RMS norm.  in_row = row_idx ? row_idx[r] : r;
 // v = x[in_row] (+ delta[in_row]); when delta is given and row_idx is not, v is
@@ -387,12 +402,60 @@ int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int
                        const int32_t* seq_slot, const int32_t* seq_start, const void* kcache,
                        const void* vcache, const int32_t* page_table, int table_stride,
                        int page_size, int ring, int n_seqs, int max_rows, int nh, int nkv, int dk,
-                       int dv, float scale, float cap, int window, void* stream);
+                       int dv, float scale, float cap, int window, const float* slopes, int chunk,
+                       const void* gate, int gate_stride, int gate_off, void* stream);
 int illm_attn_cap_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
                          const void* vcache, const int32_t* page_table, int table_stride,
                          int page_size, int ring, const int32_t* seq_slot, const int32_t* seq_len,
                          float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
-                         float scale, float cap, int window, void* stream);
+                         float scale, float cap, int window, const float* slopes, int chunk,
+                         const void* gate, int gate_stride, int gate_off, void* stream);
+// The two calls above also take: `slopes` float32 [nh] (null: none), score -= slopes[h] (i - j);
+// `chunk` > 0, a row sees only the keys j with floor(j / chunk) = floor(i / chunk); `gate` (null: none),
+// rows [., gate_stride] of the queries' dtype, out *= sigmoid(gate[row, gate_off + h dv + d]).
+// In place: q and k of rows [q (nh dk) | .. k at k_off | v at v_off] each divided by the root mean
+// square over all their heads and multiplied by qw, kw (null: untouched); v <- (1 - lam[0]) v +
+// lam[0] first[row, first_off ..] (lam null: untouched); k and v stored in the paged cache (null: not).
+int illm_qkv_norm_mix_store(void* rows, int dt, int row_len, int k_off, int v_off, const void* qw,
+                            const void* kw, int w_dt, float eps, const float* lam, const void* first,
+                            int first_stride, int first_off, const int32_t* row_pos,
+                            const int32_t* row_slot, void* kcache, void* vcache,
+                            const int32_t* page_table, int table_stride, int page_size, int ring,
+                            int T, int nh, int nkv, int dk, int dv, void* stream);
+
+// ---- what stands around the plain gated recurrence (linear_scan.hip, delta_rule.hip)
+// The scan of illm_delta_scan with a choice of rule: `correct` 1, the delta rule; 0, the plain gated
+// rule S <- diag(g) S + k (beta v)^T, o = S^T q.
+int illm_gated_scan(const float* qn, const float* kn, const float* vv, const float* beta,
+                    const float* dec, int DW, float* state, const int32_t* cu,
+                    const int32_t* seq_slot, float* o, int n_seqs, int max_rows, int G, int H, int dk,
+                    int dv, int correct, void* stream);
+// A state-space mixer's inputs from U [T, u_stride]: columns x_off.. = x (H dv) | B (G N) | C (G N)
+// through the short convolution (conv_w float32 [C, taps], conv_b [C], tail [slots, taps - 1, C] of
+// U's dtype) and SiLU into vv, kn, qn; beta = softplus(U[dt_off + h] + dt_bias[h]),
+// dec = exp(-exp(a_log[h]) beta).
+int illm_ssm_prepare(const void* U, int dt, int u_stride, int x_off, int dt_off, const float* conv_w,
+                     const float* conv_b, int taps, void* tail, const int32_t* row_slot,
+                     const float* a_log, const float* dt_bias, float* qn, float* kn, float* vv,
+                     float* beta, float* dec, int T, int G, int H, int N, int dv, int update_tail,
+                     void* stream);
+// out = rms_norm over `norm_groups` equal parts of ((o + D x) silu(Z[z_off ..])) times w.
+int illm_ssm_finish(const float* o, const float* x, const float* D, const void* Z, int z_dt,
+                    int z_stride, int z_off, const void* w, int w_dt, void* out, int out_dt, int T,
+                    int H, int dv, int norm_groups, float eps, void* stream);
+// A matrix memory's inputs from U [T, u_stride] = [q (H dk) | k (H dk) | v (H dv) | ..]: qn = q dk^-1/2,
+// kn, vv [T, H, dv + 1] (v and a column of ones); the gates i = cap tanh((U[i_off + h] + i_bias) / cap),
+// f = logsigmoid(cap tanh((U[f_off + h] + f_bias) / cap)) against the running maximum m (m_state
+// [slots, H], kept): dec = exp(f + m_before - m), beta = exp(i - m), em = exp(-m).
+int illm_memory_prepare(const void* U, int dt, int u_stride, int i_off, int f_off, const float* i_bias,
+                        const float* f_bias, float cap, float* m_state, const int32_t* cu,
+                        const int32_t* seq_slot, float* qn, float* kn, float* vv, float* beta,
+                        float* dec, float* em, int T, int n_seqs, int H, int dk, int dv, void* stream);
+// o [T, H, dv + 1] (the last column n . q): y = o / (max(|n . q|, em) + 1e-6), then per head
+// y / sqrt(mean y^2 + eps) * w[h dv + j] * sigmoid(Z[z_off + h dv + j]).
+int illm_memory_finish(const float* o, const float* em, const void* w, int w_dt, const void* Z,
+                       int z_dt, int z_stride, int z_off, void* out, int out_dt, int T, int H, int dv,
+                       float eps, void* stream);
 
 #ifdef __cplusplus
 }

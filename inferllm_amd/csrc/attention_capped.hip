@@ -1,7 +1,11 @@
 // Causal attention whose scores pass a soft cap and whose keys and values have sizes of their own:
 //     score = cap * tanh((q . k) * scale / cap)     (cap <= 0: no cap)
 // softmax over the visible keys (all j <= i, or the last `window`), context = sum p_j v_j with
-// values of width dv where queries and keys have width dk.  No position encoding is applied here.
+// values of width dv where queries and keys have width dk.  Three more things a caller may ask for:
+// a bias by distance, score -= slopes[h] (i - j) (`slopes` null: none); chunks, position i sees only
+// the keys of its own chunk, floor(j / chunk) = floor(i / chunk), counted from the sequence's
+// position 0 (`chunk` <= 0: none); an output gate, out *= sigmoid(gate[row, gate_off + h dv + d])
+// (`gate` null: none).  Positions enter through the bias and the chunks alone.
 // Keys and values live in the paged cache, K [page][kv head][row][dk], V [page][kv head][row][dv],
 // under one page table; a step first stores its rows (`kv_store2`) and then every row attends over
 // the cache at absolute positions, so whole prompts, portions of prompts and single tokens take
@@ -58,6 +62,85 @@ extern "C" int illm_kv_store2(const void* rows, int dt, int row_len, int k_off, 
     return illm_launch_status();
 }
 
+// ---------------------------------------------------------------- norms, value mixing and the store
+// rows [T, row_len] = [q (nh dk) | ... k at k_off (nkv dk) | v at v_off (nkv dv)].  In place and in
+// float32: q and k each divided by the root mean square over ALL their heads at once and multiplied
+// by a weight of that whole width (`qw`, `kw`; null: left as they are), v <- (1 - lam) v + lam first
+// with `first` [T, first_stride] + first_off the values another layer made of the same rows (`lam`
+// one float on the device; null: no mixing).  Then k and v go into the paged cache (if given).
+// grid (rows); 256 threads.
+__global__ void __launch_bounds__(256)
+qkv_norm_mix_store_kernel(void* __restrict__ rows, int dt, int row_len, int k_off, int v_off,
+                          const void* __restrict__ qw, const void* __restrict__ kw, int w_dt, float eps,
+                          const float* __restrict__ lam, const void* __restrict__ first, int first_stride,
+                          int first_off, const int32_t* __restrict__ row_pos,
+                          const int32_t* __restrict__ row_slot, void* __restrict__ kcache,
+                          void* __restrict__ vcache, const int32_t* __restrict__ page_table,
+                          int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv) {
+    __shared__ float red[16];
+    const size_t r = blockIdx.x, base = r * row_len;
+    const int pos = row_pos[r], slot = row_slot[r];
+    if (qw) {
+        const int n = nh * dk;
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < n; e += 256) { const float x = ld_f(rows, dt, base + e); ss += x * x; }
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+        for (int e = threadIdx.x; e < n; e += 256)
+            st_f(rows, dt, base + e, (ld_f(rows, dt, base + e) * inv) * ld_f(qw, w_dt, e));
+    }
+    float kinv = 1.0f;
+    if (kw) {
+        const int n = nkv * dk;
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < n; e += 256) { const float x = ld_f(rows, dt, base + k_off + e); ss += x * x; }
+        ss = block_sum(ss, red);
+        kinv = 1.0f / sqrtf(ss / (float)n + eps);
+    }
+    for (int e = threadIdx.x; e < nkv * dk; e += 256) {
+        float x = ld_f(rows, dt, base + k_off + e);
+        if (kw) {
+            x = (x * kinv) * ld_f(kw, w_dt, e);
+            st_f(rows, dt, base + k_off + e, x);
+        }
+        if (kcache) {
+            const int kvh = e / dk, d = e - kvh * dk;
+            st_f(kcache, dt, cache_row_offset(page_table, table_stride, slot, pos, page_size, ring, nkv, kvh, dk) + d, x);
+        }
+    }
+    const float l = lam ? lam[0] : 0.f;
+    for (int e = threadIdx.x; e < nkv * dv; e += 256) {
+        float x = ld_f(rows, dt, base + v_off + e);
+        if (lam) {
+            x = (1.0f - l) * x + l * ld_f(first, dt, r * first_stride + first_off + e);
+            st_f(rows, dt, base + v_off + e, x);
+        }
+        if (vcache) {
+            const int kvh = e / dv, d = e - kvh * dv;
+            st_f(vcache, dt, cache_row_offset(page_table, table_stride, slot, pos, page_size, ring, nkv, kvh, dv) + d, x);
+        }
+    }
+}
+
+extern "C" int illm_qkv_norm_mix_store(void* rows, int dt, int row_len, int k_off, int v_off,
+                                       const void* qw, const void* kw, int w_dt, float eps,
+                                       const float* lam, const void* first, int first_stride,
+                                       int first_off, const int32_t* row_pos, const int32_t* row_slot,
+                                       void* kcache, void* vcache, const int32_t* page_table,
+                                       int table_stride, int page_size, int ring, int T, int nh, int nkv,
+                                       int dk, int dv, void* stream) {
+    if (T < 0 || nh <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 || !illm_dtype_ok(dt) ||
+        !illm_dtype_ok(w_dt) || k_off < nh * dk || v_off < 0 || k_off + nkv * dk > row_len ||
+        v_off + nkv * dv > row_len || (lam && (!first || first_off < 0 || first_off + nkv * dv > first_stride)) ||
+        ((kcache == nullptr) != (vcache == nullptr)))
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(qkv_norm_mix_store_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, rows, dt,
+                       row_len, k_off, v_off, qw, kw, w_dt, eps, lam, first, first_stride, first_off, row_pos,
+                       row_slot, kcache, vcache, page_table, table_stride, page_size, ring, nh, nkv, dk, dv);
+    return illm_launch_status();
+}
+
 // ---------------------------------------------------------------- rows of a step over the cache
 // grid (query tiles, heads, sequences); 256 threads: 8 a query row.  Row r of sequence b stands at
 // position seq_start[b] + r.  q [T, q_stride] with head h at h dk.  Dynamic LDS:
@@ -68,7 +151,8 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
                      const int32_t* __restrict__ seq_start, const void* __restrict__ kcache,
                      const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                      int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
-                     float scale, float cap, int window) {
+                     float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
+                     const void* __restrict__ gate, int gate_stride, int gate_off) {
     extern __shared__ float smem[];
     const int kp = dk + 1, vp = dv + 1;
     float* qs = smem;               // [CQ][kp]
@@ -96,7 +180,10 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
     const int qrow = q0 + i, qpos = pos0 + qrow;
     const int k_hi = min(total, pos0 + q0 + CQ);
     int k_lo = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
+    if (chunk > 0) k_lo = max(k_lo, ((pos0 + q0) / chunk) * chunk);     // the block's first row sees farthest back
     k_lo = (k_lo / CK) * CK;
+    const float slope = slopes ? slopes[h] : 0.f;
+    const int c_lo = chunk > 0 ? (qpos / chunk) * chunk : 0;            // first key of this row's chunk
 
     for (int k0 = k_lo; k0 < k_hi; k0 += CK) {
         __syncthreads();
@@ -120,8 +207,8 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
             const int j = g + 8 * c, kj = k0 + j;
             float a = 0.f;
             for (int d = 0; d < dk; ++d) a = fmaf(qs[i * kp + d], ks[j * kp + d], a);
-            const bool ok = qrow < len && kj <= qpos && (window <= 0 || kj > qpos - window);
-            s[c] = ok ? soft_cap(a * scale, cap, inv_cap) : NEG_INF;
+            const bool ok = qrow < len && kj <= qpos && kj >= c_lo && (window <= 0 || kj > qpos - window);
+            s[c] = ok ? soft_cap(a * scale, cap, inv_cap) - slope * (float)(qpos - kj) : NEG_INF;
             tm = fmaxf(tm, s[c]);
         }
         tm = fmaxf(tm, __shfl_xor(tm, 1, ILLM_WAVE));
@@ -155,10 +242,15 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
     if (qrow < len) {
         const float inv = 1.0f / l_i;
         const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
+        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * dv;
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             const int d = g + 8 * k;
-            if (d < dv) st_f(out, dt, ob + d, acc[k] * inv);
+            if (d < dv) {
+                float y = acc[k] * inv;
+                if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, gb + d)));
+                st_f(out, dt, ob + d, y);
+            }
         }
     }
 }
@@ -168,7 +260,9 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
                                   const void* kcache, const void* vcache, const int32_t* page_table,
                                   int table_stride, int page_size, int ring, int n_seqs, int max_rows,
                                   int nh, int nkv, int dk, int dv, float scale, float cap, int window,
-                                  void* stream) {
+                                  const float* slopes, int chunk, const void* gate, int gate_stride,
+                                  int gate_off, void* stream) {
+    if (gate && (gate_off < 0 || gate_off + nh * dv > gate_stride)) return ILLM_ERR_ARG;
     if (n_seqs < 0 || max_rows < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 ||
         dv <= 0 || dv > 256 || page_size <= 0 || !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
@@ -180,7 +274,8 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
         return ILLM_ERR_LAUNCH;
     hipLaunchKernelGGL(attn_cap_rows_kernel, dim3((max_rows + CQ - 1) / CQ, nh, n_seqs), dim3(256), lds,
                        (hipStream_t)stream, q, q_stride, out, dt, cu, seq_slot, seq_start, kcache, vcache,
-                       page_table, table_stride, page_size, ring, nh, nkv, dk, dv, scale, cap, window);
+                       page_table, table_stride, page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes,
+                       chunk, gate, gate_stride, gate_off);
     return illm_launch_status();
 }
 
@@ -196,14 +291,17 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
                        const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                        int table_stride, int page_size, int ring, const int32_t* __restrict__ seq_slot,
                        const int32_t* __restrict__ seq_len, float* __restrict__ partial, int nsplit,
-                       int nh, int nkv, int dk, int dv, float scale, float cap, int window) {
+                       int nh, int nkv, int dk, int dv, float scale, float cap, int window,
+                       const float* __restrict__ slopes, int chunk) {
     __shared__ float wacc[4][256];
     __shared__ float wm[4], wl[4];
     const int h = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
     const int w = wave_index(), lane = threadIdx.x & 63;
     const int len = seq_len[b], slot = seq_slot[b];
     const int kvh = h / (nh / nkv);
-    const int lo_all = window > 0 ? max(0, len - window) : 0;
+    int lo_all = window > 0 ? max(0, len - window) : 0;
+    if (chunk > 0) lo_all = max(lo_all, ((len - 1) / chunk) * chunk);   // the new token's own chunk
+    const float slope = slopes ? slopes[h] : 0.f;
     const int tiles = (len + 63) / 64, t0 = lo_all / 64;
     const int per = (tiles - t0 + nsplit - 1) / nsplit;
     const int k_lo = max(lo_all, (t0 + sp * per) * 64), k_hi = min(len, (t0 + (sp + 1) * per) * 64);
@@ -244,7 +342,7 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
         float tm = NEG_INF;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            s[j] = k0 + j < k_hi ? soft_cap(s[j], cap, inv_cap) : NEG_INF;
+            s[j] = k0 + j < k_hi ? soft_cap(s[j], cap, inv_cap) - slope * (float)(len - 1 - (k0 + j)) : NEG_INF;
             tm = fmaxf(tm, s[j]);
         }
         const float m_new = fmaxf(m, tm);
@@ -285,7 +383,8 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
 
 // grid (heads, sequences): combine the splits' partial results in split order.
 __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* __restrict__ out,
-                                      int dt, int nsplit, int nh, int dv) {
+                                      int dt, int nsplit, int nh, int dv, const void* __restrict__ gate,
+                                      int gate_stride, int gate_off) {
     const int h = blockIdx.x, b = blockIdx.y;
     const float* pp = partial + ((size_t)b * nh + h) * nsplit * (dv + 2);
     float mm = NEG_INF;
@@ -302,7 +401,9 @@ __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* _
             const float ms = pp[(size_t)s * (dv + 2) + dv];
             a += (ms == NEG_INF ? 0.f : expf(ms - mm)) * pp[(size_t)s * (dv + 2) + d];
         }
-        st_f(out, dt, ((size_t)b * nh + h) * dv + d, a * inv);
+        float y = a * inv;
+        if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, (size_t)b * gate_stride + gate_off + (size_t)h * dv + d)));
+        st_f(out, dt, ((size_t)b * nh + h) * dv + d, y);
     }
 }
 
@@ -311,7 +412,9 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
                                     const int32_t* page_table, int table_stride, int page_size,
                                     int ring, const int32_t* seq_slot, const int32_t* seq_len,
                                     float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
-                                    float scale, float cap, int window, void* stream) {
+                                    float scale, float cap, int window, const float* slopes, int chunk,
+                                    const void* gate, int gate_stride, int gate_off, void* stream) {
+    if (gate && (gate_off < 0 || gate_off + nh * dv > gate_stride)) return ILLM_ERR_ARG;
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 ||
         page_size <= 0 || nsplit < 1 || nsplit > 65535 || B > 65535 || !illm_dtype_ok(dt) || !partial)
         return ILLM_ERR_ARG;
@@ -320,12 +423,13 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
     if (dt == ILLM_BF16)
         hipLaunchKernelGGL(attn_cap_decode_kernel<ILLM_BF16>, dim3(nh, B, nsplit), dim3(256), 0, st, q,
                            q_stride, kcache, vcache, page_table, table_stride, page_size, ring, seq_slot,
-                           seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window);
+                           seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk);
     else
         hipLaunchKernelGGL(attn_cap_decode_kernel<ILLM_F32>, dim3(nh, B, nsplit), dim3(256), 0, st, q,
                            q_stride, kcache, vcache, page_table, table_stride, page_size, ring, seq_slot,
-                           seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window);
+                           seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk);
     if (hipGetLastError() != hipSuccess) return ILLM_ERR_LAUNCH;
-    hipLaunchKernelGGL(attn_cap_merge_kernel, dim3(nh, B), dim3(64), 0, st, partial, out, dt, nsplit, nh, dv);
+    hipLaunchKernelGGL(attn_cap_merge_kernel, dim3(nh, B), dim3(64), 0, st, partial, out, dt, nsplit, nh, dv,
+                       gate, gate_stride, gate_off);
     return illm_launch_status();
 }

@@ -9,6 +9,10 @@
 //   delta_conv_tail the last taps - 1 inputs of every sequence, kept for the next step
 //   delta_scan      the recurrence, token after token, from the kept state and back into it
 //   delta_finish    o / rms(o) * weight * gate, gate = silu(z) or sigmoid(z)
+// The scan also runs the plain gated rule without the correction (`correct` 0),
+//     S <- diag(g) S + k (beta v)^T;   o = S^T q
+// which is the recurrence of state-space and matrix-memory mixers (linear_scan.hip prepares their
+// inputs): beta is then the weight of the token's outer product.
 // Everything but the stored projections is float32.  A sequence's rows in a step are consecutive;
 // a step may go on from any state (single tokens, portions of a prompt) or start from the zeros a
 // fresh slot holds.  Sums run in an order fixed by the sizes alone.
@@ -199,7 +203,7 @@ __device__ __forceinline__ float group_sum(float v) {
 // grid (ceil(dv / 64), H, sequences); 4 waves: a lane is a column, wave w holds rows [w NS, w NS + NS)
 // of it, so a row of S is read and written 256 bytes a wave; k, q and the decays of a row are the
 // same for a whole wave.  The waves' partial sums meet in LDS, in wave order.
-template <int NS>
+template <int NS, bool CORRECT>
 __global__ void __launch_bounds__(256)
 delta_step_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ vv, const float* __restrict__ beta,
@@ -230,9 +234,12 @@ delta_step_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
             s[ii] *= i < dk ? (DW == 1 ? dp[0] : dp[i]) : 1.f;
             pa[ii & 3] = fmaf(s[ii], kc[ii], pa[ii & 3]);
         }
-        red[0][w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
-        __syncthreads();
-        const float kv = (red[0][0][lane] + red[0][1][lane]) + (red[0][2][lane] + red[0][3][lane]);
+        float kv = 0.f;
+        if (CORRECT) {
+            red[0][w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
+            __syncthreads();
+            kv = (red[0][0][lane] + red[0][1][lane]) + (red[0][2][lane] + red[0][3][lane]);
+        }
         const float v = live ? vv[((size_t)row * H + h) * dv + col] : 0.f;
         const float u = beta[(size_t)row * H + h] * (v - kv);
         pa[0] = pa[1] = pa[2] = pa[3] = 0.f;
@@ -242,11 +249,13 @@ delta_step_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
             s[ii] = fmaf(kc[ii], u, s[ii]);
             pa[ii & 3] = fmaf(s[ii], i < dk ? qp[i] : 0.f, pa[ii & 3]);
         }
-        red[1][w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
+        // (the two buffers take turns by token where the first is not used for S^T k, so that a
+        // wave may write the next token's sums while another still reads this token's)
+        float (*rd)[64] = red[CORRECT ? 1 : (t & 1)];
+        rd[w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
         __syncthreads();
         if (w == 0 && live)
-            o[((size_t)row * H + h) * dv + col] =
-                (red[1][0][lane] + red[1][1][lane]) + (red[1][2][lane] + red[1][3][lane]);
+            o[((size_t)row * H + h) * dv + col] = (rd[0][lane] + rd[1][lane]) + (rd[2][lane] + rd[3][lane]);
     }
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii)
@@ -259,7 +268,7 @@ delta_step_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
 // registers) are issued before this chunk's arithmetic and stored after it.  One wave a block;
 // dynamic LDS: 2 * DELTA_CHUNK * 3 * 16 NS floats.
 #define DELTA_CHUNK 8
-template <int NS>
+template <int NS, bool CORRECT>
 __global__ void __launch_bounds__(64)
 delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                        const float* __restrict__ vv, const float* __restrict__ beta,
@@ -364,10 +373,13 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
                 s[ii] *= src[2 * DKP + PARTS * ii];
                 pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
             }
-            float kv = pa[0];
+            float kv = 0.f;
+            if (CORRECT) {
+                kv = pa[0];
 #pragma unroll
-            for (int a = 1; a < NA; ++a) kv += pa[a];
-            kv = group_sum<PARTS>(kv);
+                for (int a = 1; a < NA; ++a) kv += pa[a];
+                kv = group_sum<PARTS>(kv);
+            }
             const float u = cb[tt] * (cv[tt] - kv);
 #pragma unroll
             for (int a = 0; a < NA; ++a) pa[a] = 0.f;
@@ -400,10 +412,10 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
 // `max_rows`: the most rows a sequence of the step has.  It chooses the layout (16 parts from 16
 // rows on), and the layout the order of a row's sums: a row of a long step and the same row as a
 // single token differ in rounding, in nothing else.
-extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv, const float* beta,
+extern "C" int illm_gated_scan(const float* qn, const float* kn, const float* vv, const float* beta,
                                const float* dec, int DW, float* state, const int32_t* cu,
                                const int32_t* seq_slot, float* o, int n_seqs, int max_rows, int G,
-                               int H, int dk, int dv, void* stream) {
+                               int H, int dk, int dv, int correct, void* stream) {
     if (n_seqs < 0 || G <= 0 || H <= 0 || H % G || dk <= 0 || dk > 256 || dv <= 0 ||
         (DW != 1 && DW != dk) || H > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
@@ -414,28 +426,44 @@ extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv
         const size_t lds = (size_t)2 * DELTA_CHUNK * 3 * 16 * (ns <= 1 ? 1 : ns <= 2 ? 2 : ns <= 4 ? 4 : ns <= 8 ? 8 : 16) * sizeof(float);
         const dim3 grid((dv + 3) / 4, H, n_seqs);
 #define GOL(NS_)                                                                                  \
-    hipLaunchKernelGGL(delta_scan_long_kernel<NS_>, grid, dim3(64), lds, st, qn, kn, vv, beta, dec, DW, \
-                       state, cu, seq_slot, o, G, H, dk, dv)
-        if (ns <= 1) GOL(1);
-        else if (ns <= 2) GOL(2);
-        else if (ns <= 4) GOL(4);
-        else if (ns <= 8) GOL(8);
-        else GOL(16);
+    if (correct)                                                                                  \
+        hipLaunchKernelGGL((delta_scan_long_kernel<NS_, true>), grid, dim3(64), lds, st, qn, kn, vv, beta, \
+                           dec, DW, state, cu, seq_slot, o, G, H, dk, dv);                        \
+    else                                                                                          \
+        hipLaunchKernelGGL((delta_scan_long_kernel<NS_, false>), grid, dim3(64), lds, st, qn, kn, vv, beta, \
+                           dec, DW, state, cu, seq_slot, o, G, H, dk, dv)
+        if (ns <= 1) { GOL(1); }
+        else if (ns <= 2) { GOL(2); }
+        else if (ns <= 4) { GOL(4); }
+        else if (ns <= 8) { GOL(8); }
+        else { GOL(16); }
 #undef GOL
     } else {
         const int ns = (dk + 3) / 4;
         const dim3 grid((dv + 63) / 64, H, n_seqs);
 #define GOS(NS_)                                                                                  \
-    hipLaunchKernelGGL(delta_step_kernel<NS_>, grid, dim3(256), 0, st, qn, kn, vv, beta, dec, DW, state, \
-                       cu, seq_slot, o, G, H, dk, dv)
-        if (ns <= 4) GOS(4);
-        else if (ns <= 8) GOS(8);
-        else if (ns <= 16) GOS(16);
-        else if (ns <= 32) GOS(32);
-        else GOS(64);
+    if (correct)                                                                                  \
+        hipLaunchKernelGGL((delta_step_kernel<NS_, true>), grid, dim3(256), 0, st, qn, kn, vv, beta, dec, \
+                           DW, state, cu, seq_slot, o, G, H, dk, dv);                             \
+    else                                                                                          \
+        hipLaunchKernelGGL((delta_step_kernel<NS_, false>), grid, dim3(256), 0, st, qn, kn, vv, beta, dec, \
+                           DW, state, cu, seq_slot, o, G, H, dk, dv)
+        if (ns <= 4) { GOS(4); }
+        else if (ns <= 8) { GOS(8); }
+        else if (ns <= 16) { GOS(16); }
+        else if (ns <= 32) { GOS(32); }
+        else { GOS(64); }
 #undef GOS
     }
     return illm_launch_status();
+}
+
+extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv, const float* beta,
+                               const float* dec, int DW, float* state, const int32_t* cu,
+                               const int32_t* seq_slot, float* o, int n_seqs, int max_rows, int G,
+                               int H, int dk, int dv, void* stream) {
+    return illm_gated_scan(qn, kn, vv, beta, dec, DW, state, cu, seq_slot, o, n_seqs, max_rows, G, H, dk,
+                           dv, 1, stream);
 }
 
 // grid (rows, H); one wave: out[r, h dv + j] = o / sqrt(mean_j o^2 + eps) * w[j] * act(z[r, h dv + j]),

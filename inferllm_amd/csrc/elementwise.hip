@@ -37,6 +37,78 @@ extern "C" int illm_embed(const int32_t* tokens, const void* table, int table_dt
     return illm_embed_scaled(tokens, table, table_dt, out, T, E, V, 1.0f, stream);
 }
 
+// Token row times a scale, plus a row of a table hashed by the pair (previous token, token), plus a
+// learned row of the position:
+//     out = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets] + places[pos]
+// A sequence's first token (position 0) takes row `buckets` of `pairs`, its last.  The token before a
+// row is the row above it if that belongs to the same slot, else `last_token[slot]`: what the
+// sequence's last step left.  `pairs` or `places` may be null (that addend is left out).
+// `remember`: every sequence brings one row, and the row's thread also leaves its token in
+// `last_token`; steps of several rows a sequence call illm_remember_last afterwards.
+__global__ void embed_pairs_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ row_pos,
+                                   const int32_t* __restrict__ row_slot, const void* __restrict__ table,
+                                   int table_dt, const void* __restrict__ pairs, int pairs_dt,
+                                   const void* __restrict__ places, int places_dt,
+                                   int32_t* __restrict__ last_token, float* __restrict__ out, int E, int V,
+                                   int buckets, int mul_prev, int mul_cur, int n_places, float scale,
+                                   int remember) {
+    const int t = blockIdx.x;
+    int id = tokens[t];
+    id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+    int pos = row_pos[t];
+    pos = pos < 0 ? 0 : (pos >= n_places ? n_places - 1 : pos);
+    const int slot = row_slot[t];
+    int pair = buckets;
+    if (pairs && row_pos[t] > 0) {
+        int prev = (t > 0 && row_slot[t - 1] == slot) ? tokens[t - 1] : last_token[slot];
+        prev = prev < 0 ? 0 : (prev >= V ? V - 1 : prev);
+        pair = (int)(((long long)prev * mul_prev + (long long)id * mul_cur) % buckets);
+    }
+    const size_t src = (size_t)id * E, dst = (size_t)t * E;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) {
+        float v = ld_f(table, table_dt, src + i) * scale;
+        if (pairs) v += ld_f(pairs, pairs_dt, (size_t)pair * E + i);
+        if (places) v += ld_f(places, places_dt, (size_t)pos * E + i);
+        out[dst + i] = v;
+    }
+    if (remember && last_token && threadIdx.x == 0) last_token[slot] = id;
+}
+
+extern "C" int illm_embed_pairs(const int32_t* tokens, const int32_t* row_pos, const int32_t* row_slot,
+                                const void* table, int table_dt, const void* pairs, int pairs_dt,
+                                const void* places, int places_dt, int32_t* last_token, float* out,
+                                int T, int E, int V, int buckets, int mul_prev, int mul_cur,
+                                int n_places, float scale, int remember, void* stream) {
+    if (T < 0 || E <= 0 || V <= 0 || !illm_dtype_ok(table_dt) || (pairs && (!illm_dtype_ok(pairs_dt) ||
+        buckets <= 0 || mul_prev < 0 || mul_cur < 0 || !last_token)) || (places && (!illm_dtype_ok(places_dt) ||
+        n_places <= 0)))
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(embed_pairs_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, tokens, row_pos,
+                       row_slot, table, table_dt, pairs, pairs_dt, places, places_dt, last_token, out, E, V,
+                       buckets, mul_prev, mul_cur, places ? n_places : 1, scale, remember);
+    return illm_launch_status();
+}
+
+// last_token[seq_slot[b]] = the last token of sequence b's rows in this step (none: left as it is).
+__global__ void remember_last_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ cu,
+                                     const int32_t* __restrict__ seq_slot, int32_t* __restrict__ last_token,
+                                     int n_seqs) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= n_seqs) return;
+    const int end = cu[b + 1];
+    if (end > cu[b]) last_token[seq_slot[b]] = tokens[end - 1];
+}
+
+extern "C" int illm_remember_last(const int32_t* tokens, const int32_t* cu, const int32_t* seq_slot,
+                                  int32_t* last_token, int n_seqs, void* stream) {
+    if (n_seqs < 0) return ILLM_ERR_ARG;
+    if (n_seqs == 0) return ILLM_OK;
+    hipLaunchKernelGGL(remember_last_kernel, dim3((n_seqs + 63) / 64), dim3(64), 0, (hipStream_t)stream,
+                       tokens, cu, seq_slot, last_token, n_seqs);
+    return illm_launch_status();
+}
+
 // ---------------------------------------------------------------- sums and activations by element
 __global__ void sum_rows_kernel(const void* __restrict__ a, int a_dt, const void* __restrict__ b,
                                 int b_dt, float* __restrict__ out, size_t n) {
@@ -81,6 +153,22 @@ extern "C" int illm_relu_squared(const void* x, void* out, int dt, size_t n, voi
     if (!illm_dtype_ok(dt)) return ILLM_ERR_ARG;
     if (n == 0) return ILLM_OK;
     hipLaunchKernelGGL(relu_squared_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, x, out, dt, n);
+    return illm_launch_status();
+}
+
+// 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), the tanh form of GELU.
+__global__ void gelu_tanh_kernel(const void* __restrict__ x, void* __restrict__ out, int dt, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float z = ld_f(x, dt, i);
+    st_f(out, dt, i, 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))));
+}
+
+extern "C" int illm_gelu_tanh(const void* x, void* out, int dt, size_t n, void* stream) {
+    if (!illm_dtype_ok(dt)) return ILLM_ERR_ARG;
+    if (n == 0) return ILLM_OK;
+    hipLaunchKernelGGL(gelu_tanh_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, x, out, dt, n);
     return illm_launch_status();
 }

@@ -1,0 +1,245 @@
+// What stands around the plain gated recurrence (illm_gated_scan with `correct` 0,
+//     S <- g S + k (beta v)^T;   o = S^T q,   S [key dim, value dim] float32 per head)
+// for two mixers that keep such a state.
+//
+// A state-space mixer with a scalar decay a head (state-space duality):
+//   ssm_prepare   short causal convolution with bias over time of the x | B | C columns of the input
+//                 projection (the taps before a step's first row from the kept tail), SiLU;
+//                 dt = softplus(dt + dt_bias), g = exp(-exp(A_log) dt), beta = dt; k = B, q = C of the
+//                 head's group, v = x
+//   ssm_finish    y = (o + D x) silu(z), RMS norm in `norm_groups` equal parts of the row, weight
+//
+// A matrix memory with exponential gates held in range by a running maximum m (from 0):
+//   memory_rows   q dim^-1/2, k, and v with a column of ones behind it as float32 (the state's
+//                 last column is then the normaliser n = sum of the weighted keys)
+//   memory_gates  i = cap tanh((i + b_i) / cap), f = logsigmoid(cap tanh((f + b_f) / cap)),
+//                 m_t = max(f + m_(t-1), i), g = exp(f + m_(t-1) - m_t), beta = exp(i - m_t), token
+//                 after token per sequence and head, m kept per sequence
+//   memory_finish o / (max(|n . q|, exp(-m)) + 1e-6), RMS norm per head, weight, sigmoid gate
+//
+// Everything but the stored projections is float32.  A sequence's rows in a step are consecutive.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define SCAN_MAX_TAPS 8
+
+__device__ __forceinline__ float ls_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float ls_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float ls_log_sigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+// ---------------------------------------------------------------- state-space mixer
+// grid (rows, NB); 256 threads over the convolution's channels.  U [T, u_stride]: columns
+// [x_off, x_off + C) = x (H dv) | B (G N) | C (G N) before the convolution, dt_off: H columns.
+// `update_tail`: every sequence brings one row, and the thread that has read a channel's taps also
+// writes its tail for the next step.
+__global__ void __launch_bounds__(256)
+ssm_prepare_kernel(const void* __restrict__ U, int dt, int u_stride, int x_off, int dt_off,
+                   const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps,
+                   void* __restrict__ tail, const int32_t* __restrict__ row_slot,
+                   const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                   float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
+                   float* __restrict__ beta, float* __restrict__ dec, int G, int H, int N, int dv,
+                   int update_tail) {
+    const int r = blockIdx.x, NB = gridDim.y;
+    const int inner = H * dv, GN = G * N, C = inner + 2 * GN, K = taps - 1;
+    const int slot = row_slot[r];
+    int before = 0;                                     // rows of this sequence ahead of r in the step, up to K
+    while (before < K && r - before - 1 >= 0 && row_slot[r - before - 1] == slot) ++before;
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * NB) {
+        float x[SCAN_MAX_TAPS], cw[SCAN_MAX_TAPS];
+#pragma unroll
+        for (int j = 0; j < SCAN_MAX_TAPS; ++j) {
+            x[j] = cw[j] = 0.f;
+            if (j < taps) {
+                const int d = K - j;                    // tap j looks d tokens back
+                x[j] = d <= before ? ld_f(U, dt, (size_t)(r - d) * u_stride + x_off + c)
+                                   : ld_f(tail, dt, ((size_t)slot * K + (K - (d - before))) * C + c);
+                cw[j] = conv_w[(size_t)c * taps + j];
+            }
+        }
+        float a = conv_b[c];
+#pragma unroll
+        for (int j = 0; j < SCAN_MAX_TAPS; ++j) {
+            if (j < taps) {
+                a = fmaf(cw[j], x[j], a);
+                if (update_tail && j > 0) st_f(tail, dt, ((size_t)slot * K + (j - 1)) * C + c, x[j]);
+            }
+        }
+        const float y = a * ls_sigmoid(a);
+        if (c < inner) vv[(size_t)r * inner + c] = y;
+        else if (c < inner + GN) kn[(size_t)r * GN + (c - inner)] = y;
+        else qn[(size_t)r * GN + (c - inner - GN)] = y;
+    }
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < H; i += 256 * NB) {
+        const float step = ls_softplus(ld_f(U, dt, (size_t)r * u_stride + dt_off + i) + dt_bias[i]);
+        beta[(size_t)r * H + i] = step;
+        dec[(size_t)r * H + i] = expf(-expf(a_log[i]) * step);
+    }
+}
+
+extern "C" int illm_ssm_prepare(const void* U, int dt, int u_stride, int x_off, int dt_off,
+                                const float* conv_w, const float* conv_b, int taps, void* tail,
+                                const int32_t* row_slot, const float* a_log, const float* dt_bias,
+                                float* qn, float* kn, float* vv, float* beta, float* dec, int T, int G,
+                                int H, int N, int dv, int update_tail, void* stream) {
+    if (T < 0 || G <= 0 || H <= 0 || H % G || N <= 0 || dv <= 0 || taps < 1 || taps > SCAN_MAX_TAPS ||
+        !illm_dtype_ok(dt) || x_off < 0 || dt_off < 0 || x_off + H * dv + 2 * G * N > u_stride ||
+        dt_off + H > u_stride)
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    const int C = H * dv + 2 * G * N, most = (C + 255) / 256;
+    int nb = T >= 2048 ? 1 : (2048 + T - 1) / T;        // enough blocks to fill the chip when the rows are few
+    nb = nb > most ? most : nb;
+    hipLaunchKernelGGL(ssm_prepare_kernel, dim3(T, nb), dim3(256), 0, (hipStream_t)stream, U, dt, u_stride,
+                       x_off, dt_off, conv_w, conv_b, taps, tail, row_slot, a_log, dt_bias, qn, kn, vv,
+                       beta, dec, G, H, N, dv, update_tail);
+    return illm_launch_status();
+}
+
+// grid (rows, norm groups); 256 threads.  y_j = (o_j + D[head of j] x_j) silu(z_j) over the part's
+// columns, out = y / sqrt(mean over the part of y^2 + eps) * w.  Z [T, z_stride] + z_off.
+__global__ void __launch_bounds__(256)
+ssm_finish_kernel(const float* __restrict__ o, const float* __restrict__ x,
+                  const float* __restrict__ D, const void* __restrict__ Z, int z_dt, int z_stride,
+                  int z_off, const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
+                  int inner, int dv, int part, float eps) {
+    __shared__ float red[16];
+    const size_t r = blockIdx.x;
+    const int j0 = blockIdx.y * part;
+    float ss = 0.f;
+    for (int j = j0 + threadIdx.x; j < j0 + part; j += 256) {
+        const float z = ld_f(Z, z_dt, r * z_stride + z_off + j);
+        const float y = fmaf(D[j / dv], x[r * inner + j], o[r * inner + j]) * (z * ls_sigmoid(z));
+        ss += y * y;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)part + eps);
+    for (int j = j0 + threadIdx.x; j < j0 + part; j += 256) {
+        const float z = ld_f(Z, z_dt, r * z_stride + z_off + j);
+        const float y = fmaf(D[j / dv], x[r * inner + j], o[r * inner + j]) * (z * ls_sigmoid(z));
+        st_f(out, out_dt, r * inner + j, (y * inv) * ld_f(w, w_dt, j));
+    }
+}
+
+extern "C" int illm_ssm_finish(const float* o, const float* x, const float* D, const void* Z, int z_dt,
+                               int z_stride, int z_off, const void* w, int w_dt, void* out, int out_dt,
+                               int T, int H, int dv, int norm_groups, float eps, void* stream) {
+    if (T < 0 || H <= 0 || dv <= 0 || norm_groups <= 0 || norm_groups > 65535 ||
+        (H * dv) % norm_groups || !illm_dtype_ok(z_dt) || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
+        z_off < 0 || z_off + H * dv > z_stride)
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(ssm_finish_kernel, dim3(T, norm_groups), dim3(256), 0, (hipStream_t)stream, o, x, D,
+                       Z, z_dt, z_stride, z_off, w, w_dt, out, out_dt, H * dv, dv, (H * dv) / norm_groups, eps);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- matrix memory
+// grid (rows); 256 threads.  U [T, u_stride] = [q (H dk) | k (H dk) | v (H dv) | ...].
+__global__ void __launch_bounds__(256)
+memory_rows_kernel(const void* __restrict__ U, int dt, int u_stride, float* __restrict__ qn,
+                   float* __restrict__ kn, float* __restrict__ vv, int H, int dk, int dv, float qscale) {
+    const size_t r = blockIdx.x;
+    const int nq = H * dk, nv = H * (dv + 1);
+    for (int i = threadIdx.x; i < nq; i += 256) {
+        qn[r * nq + i] = ld_f(U, dt, r * u_stride + i) * qscale;
+        kn[r * nq + i] = ld_f(U, dt, r * u_stride + nq + i);
+    }
+    for (int i = threadIdx.x; i < nv; i += 256) {
+        const int h = i / (dv + 1), j = i - h * (dv + 1);
+        vv[r * nv + i] = j < dv ? ld_f(U, dt, r * u_stride + 2 * nq + h * dv + j) : 1.0f;
+    }
+}
+
+// grid (sequences, H); one wave.  64 tokens at a time: every lane forms its token's two gates, then
+// the running maximum goes through the 64 tokens in order (the lanes' values are read one after the
+// other as scalars), and every lane leaves its token's decay, weight and exp(-m).
+__global__ void __launch_bounds__(64)
+memory_gates_kernel(const void* __restrict__ U, int dt, int u_stride, int i_off, int f_off,
+                    const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                    float* __restrict__ m_state, const int32_t* __restrict__ cu,
+                    const int32_t* __restrict__ seq_slot, float* __restrict__ beta,
+                    float* __restrict__ dec, float* __restrict__ em, int H) {
+    const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    if (n <= 0) return;
+    const int slot = seq_slot[b];
+    const float bi = i_bias[h], bf = f_bias[h], inv_cap = 1.0f / cap;
+    float m = m_state[(size_t)slot * H + h];
+    for (int t0 = 0; t0 < n; t0 += 64) {
+        const bool ok = t0 + lane < n;
+        const size_t row = (size_t)(r0 + (ok ? t0 + lane : n - 1));
+        const float ig = ok ? cap * tanhf((ld_f(U, dt, row * u_stride + i_off + h) + bi) * inv_cap) : -INFINITY;
+        const float fg = ok ? ls_log_sigmoid(cap * tanhf((ld_f(U, dt, row * u_stride + f_off + h) + bf) * inv_cap)) : 0.f;
+        float m_before = 0.f, m_mine = 0.f;
+#pragma unroll
+        for (int l = 0; l < 64; ++l) {
+            const float fl = __shfl(fg, l, 64), il = __shfl(ig, l, 64);
+            const float m_new = fmaxf(fl + m, il);      // a lane beyond the sequence leaves m as it is
+            if (lane == l) { m_before = m; m_mine = m_new; }
+            m = m_new;
+        }
+        if (ok) {
+            dec[row * H + h] = expf(fg + m_before - m_mine);
+            beta[row * H + h] = expf(ig - m_mine);
+            em[row * H + h] = expf(-m_mine);
+        }
+    }
+    if (lane == 0) m_state[(size_t)slot * H + h] = m;
+}
+
+extern "C" int illm_memory_prepare(const void* U, int dt, int u_stride, int i_off, int f_off,
+                                   const float* i_bias, const float* f_bias, float cap, float* m_state,
+                                   const int32_t* cu, const int32_t* seq_slot, float* qn, float* kn,
+                                   float* vv, float* beta, float* dec, float* em, int T, int n_seqs,
+                                   int H, int dk, int dv, void* stream) {
+    if (T < 0 || n_seqs < 0 || n_seqs > 65535 || H <= 0 || H > 65535 || dk <= 0 || dv <= 0 ||
+        !illm_dtype_ok(dt) || !(cap > 0.f) || 2 * H * dk + H * dv > u_stride || i_off < 0 || f_off < 0 ||
+        i_off + H > u_stride || f_off + H > u_stride)
+        return ILLM_ERR_ARG;
+    if (T == 0 || n_seqs == 0) return ILLM_OK;
+    hipLaunchKernelGGL(memory_rows_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, U, dt, u_stride, qn,
+                       kn, vv, H, dk, dv, 1.0f / sqrtf((float)dk));
+    if (hipGetLastError() != hipSuccess) return ILLM_ERR_LAUNCH;
+    hipLaunchKernelGGL(memory_gates_kernel, dim3(n_seqs, H), dim3(64), 0, (hipStream_t)stream, U, dt,
+                       u_stride, i_off, f_off, i_bias, f_bias, cap, m_state, cu, seq_slot, beta, dec, em, H);
+    return illm_launch_status();
+}
+
+// grid (rows, H); one wave.  o [T, H, dv + 1]: the last column is n . q.
+//   y_j = o_j / (max(|n . q|, exp(-m)) + 1e-6);  out = y / sqrt(mean_j y^2 + eps) * w[h dv + j] * sigmoid(z)
+__global__ void __launch_bounds__(64)
+memory_finish_kernel(const float* __restrict__ o, const float* __restrict__ em,
+                     const void* __restrict__ w, int w_dt, const void* __restrict__ Z, int z_dt,
+                     int z_stride, int z_off, void* __restrict__ out, int out_dt, int H, int dv, float eps) {
+    const size_t r = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const float* op = o + (r * H + h) * (dv + 1);
+    const float den = fmaxf(fabsf(op[dv]), em[r * H + h]) + 1e-6f;
+    float ss = 0.f;
+    for (int j = lane; j < dv; j += 64) {
+        const float y = op[j] / den;
+        ss += y * y;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+    for (int j = lane; j < dv; j += 64) {
+        const float z = ld_f(Z, z_dt, r * z_stride + z_off + (size_t)h * dv + j);
+        st_f(out, out_dt, (r * H + h) * dv + j,
+             ((op[j] / den) * inv) * ld_f(w, w_dt, (size_t)h * dv + j) * ls_sigmoid(z));
+    }
+}
+
+extern "C" int illm_memory_finish(const float* o, const float* em, const void* w, int w_dt, const void* Z,
+                                  int z_dt, int z_stride, int z_off, void* out, int out_dt, int T, int H,
+                                  int dv, float eps, void* stream) {
+    if (T < 0 || H <= 0 || H > 65535 || dv <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(z_dt) ||
+        !illm_dtype_ok(out_dt) || z_off < 0 || z_off + H * dv > z_stride)
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(memory_finish_kernel, dim3(T, H), dim3(64), 0, (hipStream_t)stream, o, em, w, w_dt, Z,
+                       z_dt, z_stride, z_off, out, out_dt, H, dv, eps);
+    return illm_launch_status();
+}

@@ -104,7 +104,12 @@ class DecoderModel:
         return out
 
     def state_lines(self) -> Dict[int, StateSpec]:
+        """Fixed-size state per sequence by cache line; an embedding that keeps state of its own
+        (the token before a step's first) has it under the line it names (`STATE_LINE`)."""
         out: Dict[int, StateSpec] = {}
+        own = getattr(self.embedding, "state_spec", lambda: None)()
+        if own is not None:
+            out[self.embedding.STATE_LINE] = own
         for e in self.schedule:
             spec = self.layers[e.layer].mixer.state_spec()
             if spec is not None:

@@ -114,6 +114,43 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float = 1.0, copies:
     return out
 
 
+def embed_pairs(tokens: torch.Tensor, row_pos: torch.Tensor, row_slot: torch.Tensor,
+                table: torch.Tensor, scale: float, pairs: Optional[torch.Tensor], buckets: int,
+                mul_prev: int, mul_cur: int, places: Optional[torch.Tensor],
+                last_token: Optional[torch.Tensor], remember: bool) -> torch.Tensor:
+    """float32 [T, E]: table[token] * scale + pairs[(prev * mul_prev + token * mul_cur) mod buckets]
+    + places[position].  prev is the row above if it belongs to the same slot, else
+    `last_token[slot]` (int32 [slots]); a row at position 0 takes `pairs[buckets]`.  `pairs`
+    [buckets + 1, E] and `places` [positions, E] may be None.  `remember` (every sequence brings one
+    row): the row's token is left in `last_token` too; otherwise `remember_last` does that."""
+    _gpu(tokens, row_pos, row_slot, table, pairs, places, last_token)
+    T = tokens.numel()
+    _i32(tokens); _i32(row_pos, T); _i32(row_slot, T); _i32(last_token)
+    _need(table.dim() == 2, "embed_pairs: table [V, E]")
+    V, E = table.shape
+    if pairs is not None:
+        _need(pairs.shape == (buckets + 1, E) and last_token is not None,
+              f"embed_pairs: pairs [{buckets + 1}, {E}] and the slots' last tokens")
+    _need(places is None or (places.dim() == 2 and places.shape[1] == E), "embed_pairs: places [positions, E]")
+    out = torch.empty((T, E), dtype=torch.float32, device=table.device)
+    _check(_lib().illm_embed_pairs(
+        _p(tokens), _p(row_pos), _p(row_slot), _p(table), _code(table), _p(pairs),
+        _code(pairs) if pairs is not None else 0, _p(places), _code(places) if places is not None else 0,
+        _p(last_token), _p(out), T, E, V, int(buckets), int(mul_prev), int(mul_cur),
+        places.shape[0] if places is not None else 1, ctypes.c_float(scale), 1 if remember else 0,
+        _stream()), "embed_pairs")
+    return out
+
+
+def remember_last(tokens: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+                  last_token: torch.Tensor, n_seqs: int) -> None:
+    """last_token[seq_slot[b]] = the last of sequence b's tokens in this step."""
+    _gpu(tokens, cu_seqlens, seq_slot, last_token)
+    _i32(tokens); _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(last_token)
+    _check(_lib().illm_remember_last(_p(tokens), _p(cu_seqlens), _p(seq_slot), _p(last_token), n_seqs,
+                                     _stream()), "remember_last")
+
+
 def sum_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """float32(a) + float32(b), element by element: what a block whose mixer and feed-forward
     read the same rows leaves for the residual stream."""
@@ -149,6 +186,15 @@ def relu_squared(x: torch.Tensor) -> torch.Tensor:
     out = torch.empty_like(x)
     _check(_lib().illm_relu_squared(_p(x), _p(out), _code(x), ctypes.c_size_t(x.numel()), _stream()),
            "relu_squared")
+    return out
+
+
+def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))), element by element."""
+    _gpu(x)
+    out = torch.empty_like(x)
+    _check(_lib().illm_gelu_tanh(_p(x), _p(out), _code(x), ctypes.c_size_t(x.numel()), _stream()),
+           "gelu_tanh")
     return out
 
 
@@ -1450,15 +1496,63 @@ def _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, wha
           and page_table.dim() == 2, f"{what}: cache shape or dtype")
 
 
+def _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, what):
+    _gpu(slopes, gate)
+    _need(slopes is None or (slopes.dtype == torch.float32 and slopes.shape == (nh,)),
+          f"{what}: slopes float32 [{nh}]")
+    _need(gate is None or (gate.dim() == 2 and gate.dtype == q.dtype and gate.shape[0] == q.shape[0]
+                           and 0 <= gate_off and gate_off + nh * dv <= gate.shape[1]),
+          f"{what}: gate rows of the queries' dtype with {nh * dv} columns from {gate_off}")
+
+
+def qkv_norm_mix_store(rows: torch.Tensor, k_off: int, v_off: int, q_weight: Optional[torch.Tensor],
+                       k_weight: Optional[torch.Tensor], eps: float, lam: Optional[torch.Tensor],
+                       first: Optional[torch.Tensor], first_off: int, row_pos: torch.Tensor,
+                       row_slot: torch.Tensor, kcache: Optional[torch.Tensor],
+                       vcache: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+                       page_size: int, ring: int, nh: int, nkv: int, dk: int, dv: int) -> None:
+    """In place on packed rows [q (nh dk) | .. k at k_off (nkv dk) | v at v_off (nkv dv)], in float32:
+    q and k each divided by the root mean square over all their heads at once and multiplied by
+    `q_weight` [nh dk], `k_weight` [nkv dk] (None: untouched); v <- (1 - lam) v + lam first[:,
+    first_off ..] with `lam` one float32 on the device (None: untouched); then k and v are stored in
+    the paged cache K [pages, nkv, page_size, dk], V [pages, nkv, page_size, dv] (None: not stored)."""
+    _gpu(rows, q_weight, k_weight, lam, first, row_pos, row_slot, kcache, vcache, page_table)
+    T = rows.shape[0]
+    _i32(row_pos, T); _i32(row_slot, T); _i32(page_table)
+    _need(rows.dim() == 2, "qkv_norm_mix_store: rows [T, n]")
+    _need((q_weight is None) == (k_weight is None), "qkv_norm_mix_store: both norm weights or none")
+    if q_weight is not None:
+        _need(q_weight.shape == (nh * dk,) and k_weight.shape == (nkv * dk,) and q_weight.dtype == k_weight.dtype,
+              "qkv_norm_mix_store: norm weights over all heads")
+    if lam is not None:
+        _need(lam.dtype == torch.float32 and lam.numel() == 1 and first is not None and first.dim() == 2
+              and first.dtype == rows.dtype and first.shape[0] == T and first_off + nkv * dv <= first.shape[1],
+              "qkv_norm_mix_store: lam float32 [1] and the first layer's rows")
+    if kcache is not None:
+        _need(kcache.dtype == rows.dtype and vcache.dtype == rows.dtype
+              and kcache.shape[1:] == (nkv, page_size, dk) and vcache.shape[1:] == (nkv, page_size, dv)
+              and page_table is not None and page_table.dim() == 2, "qkv_norm_mix_store: cache shapes")
+    _check(_lib().illm_qkv_norm_mix_store(
+        _p(rows), _code(rows), rows.shape[1], k_off, v_off, _p(q_weight), _p(k_weight),
+        _code(q_weight) if q_weight is not None else 0, ctypes.c_float(eps), _p(lam), _p(first),
+        first.shape[1] if first is not None else 0, first_off, _p(row_pos), _p(row_slot), _p(kcache),
+        _p(vcache), _p(page_table), page_table.shape[1] if page_table is not None else 0, page_size, ring,
+        T, nh, nkv, dk, dv, _stream()), "qkv_norm_mix_store")
+
+
 def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
                   seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                   page_table: torch.Tensor, page_size: int, ring: int, n_seqs: int, max_rows: int,
                   nh: int, nkv: int, dk: int, dv: int, scale: float, cap: float,
-                  window: int) -> torch.Tensor:
+                  window: int, slopes: Optional[torch.Tensor] = None, chunk: int = 0,
+                  gate: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
     """Causal attention of a step's packed rows over the paged cache (which holds the step's own
     keys and values by now): row r of sequence b stands at position seq_start[b] + r; scores
     cap tanh(q . k scale / cap) (cap 0: none); queries and keys of width dk, values of dv.
+    `slopes` float32 [nh]: score -= slopes[h] (i - j).  `chunk` > 0: a row sees only the keys of its
+    own chunk of positions.  `gate` [T, n] (columns gate_off ..): out *= sigmoid(gate).
     Returns [T, nh dv]."""
+    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_rows")
     _gpu(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
     _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_rows")
@@ -1466,7 +1560,8 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
     _check(_lib().illm_attn_cap_rows(
         _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh, nkv,
-        dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
+        dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk), _p(gate),
+        gate.shape[1] if gate is not None else 0, gate_off, _stream()),
         f"attn_cap_rows (sizes {dk}, {dv})")
     return out
 
@@ -1474,9 +1569,11 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
 def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                     page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
                     seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
-                    cap: float, window: int, nsplit: int) -> torch.Tensor:
+                    cap: float, window: int, nsplit: int, slopes: Optional[torch.Tensor] = None,
+                    chunk: int = 0, gate: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
     """The same attention for one new token per sequence: row b of q against the seq_len[b] keys
     (the new one included) of its slot, the keys cut into `nsplit` ranges.  Returns [B, nh dv]."""
+    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_decode")
     _gpu(q, kcache, vcache, page_table, seq_slot, seq_len)
     B = q.shape[0]
     _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
@@ -1486,7 +1583,8 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     _check(_lib().illm_attn_cap_decode(
         _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(page_table),
         page_table.shape[1], page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh,
-        nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
+        nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk),
+        _p(gate), gate.shape[1] if gate is not None else 0, gate_off, _stream()),
         f"attn_cap_decode (sizes {dk}, {dv})")
     return out
 
@@ -1532,21 +1630,25 @@ def delta_prepare(P: torch.Tensor, b_off: int, A: torch.Tensor, a_off: int, conv
 
 
 def delta_conv_tail(P: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
-                    seq_slot: torch.Tensor, n_seqs: int, taps: int) -> None:
-    """Keep the last taps - 1 convolution inputs of every sequence of the step in `tail`."""
+                    seq_slot: torch.Tensor, n_seqs: int, taps: int, col_off: int = 0) -> None:
+    """Keep the last taps - 1 convolution inputs of every sequence of the step in `tail`; the
+    convolution's channels are P's columns from `col_off` on."""
     _gpu(P, tail, cu_seqlens, seq_slot)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
     C = tail.shape[2]
-    _need(P.dim() == 2 and P.shape[1] >= C and tail.shape[1] == max(taps - 1, 1), "delta_conv_tail: shapes")
-    _check(_lib().illm_delta_conv_tail(_p(P), _code(P), P.shape[1], _p(tail), _code(tail),
+    _need(P.dim() == 2 and col_off >= 0 and P.shape[1] >= col_off + C
+          and tail.shape[1] == max(taps - 1, 1), "delta_conv_tail: shapes")
+    first = ctypes.c_void_p(P.data_ptr() + col_off * P.element_size())
+    _check(_lib().illm_delta_conv_tail(first, _code(P), P.shape[1], _p(tail), _code(tail),
                                        _p(cu_seqlens), _p(seq_slot), n_seqs, C, taps, _stream()),
            "delta_conv_tail")
 
 
 def delta_scan(qn, kn, vv, beta, dec, state: torch.Tensor, cu_seqlens: torch.Tensor,
-               seq_slot: torch.Tensor, n_seqs: int, max_rows: int) -> torch.Tensor:
+               seq_slot: torch.Tensor, n_seqs: int, max_rows: int, correct: bool = True) -> torch.Tensor:
     """The recurrence S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q over every
-    sequence's rows in order, from `state` float32 [slots, H, dk, dv] and back into it.
+    sequence's rows in order, from `state` float32 [slots, H, dk, dv] and back into it.  With
+    `correct` False the plain gated rule, u = beta v: S <- diag(g) S + k (beta v)^T.
     `max_rows`: the most rows a sequence brings (long sequences are laid out for their chain of
     tokens, short steps for the state's bytes).  Returns o float32 [T, H, dv]."""
     _gpu(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot)
@@ -1557,11 +1659,112 @@ def delta_scan(qn, kn, vv, beta, dec, state: torch.Tensor, cu_seqlens: torch.Ten
     _need(kn.shape == qn.shape and beta.shape == (T, H) and dec.shape[:2] == (T, H)
           and dec.shape[2] in (1, dk) and state.shape[1:] == (H, dk, dv), "delta_scan: shapes")
     o = torch.empty((T, H, dv), dtype=torch.float32, device=qn.device)
-    _check(_lib().illm_delta_scan(_p(qn), _p(kn), _p(vv), _p(beta), _p(dec), dec.shape[2], _p(state),
+    _check(_lib().illm_gated_scan(_p(qn), _p(kn), _p(vv), _p(beta), _p(dec), dec.shape[2], _p(state),
                                   _p(cu_seqlens), _p(seq_slot), _p(o), n_seqs, max_rows, G, H, dk, dv,
-                                  _stream()),
+                                  1 if correct else 0, _stream()),
            "delta_scan")
     return o
+
+
+# ------------------------------------------------------------------ around the plain gated rule
+def ssm_prepare(U: torch.Tensor, x_off: int, dt_off: int, conv_w: torch.Tensor, conv_b: torch.Tensor,
+                tail: torch.Tensor, row_slot: torch.Tensor, a_log: torch.Tensor,
+                dt_bias: torch.Tensor, G: int, H: int, N: int, dv: int, update_tail: bool = False):
+    """A state-space mixer's float32 inputs for the plain gated rule, from the input projection U
+    [T, n]: columns x_off .. = x (H dv) | B (G N) | C (G N) go through the short convolution with
+    bias (conv_w float32 [C, taps], conv_b [C]; the inputs before a step's first row from `tail`
+    [slots, taps - 1, C]) and SiLU; step = softplus(U[:, dt_off + h] + dt_bias[h]) is the token's
+    weight and exp(-exp(a_log[h]) step) its decay.  `update_tail` as in `delta_prepare`.
+    Returns (q = C [T, G, N], k = B [T, G, N], v = x [T, H, dv], weight [T, H], decay [T, H, 1])."""
+    _gpu(U, conv_w, conv_b, tail, row_slot, a_log, dt_bias)
+    T = U.shape[0]
+    _i32(row_slot, T)
+    C = H * dv + 2 * G * N
+    _need(U.dim() == 2 and U.shape[1] >= max(x_off + C, dt_off + H), "ssm_prepare: projection too narrow")
+    _need(conv_w.dtype == torch.float32 and conv_w.dim() == 2 and conv_w.shape[0] == C
+          and conv_b.dtype == torch.float32 and conv_b.shape == (C,), "ssm_prepare: conv_w float32 [C, taps], conv_b [C]")
+    taps = conv_w.shape[1]
+    _need(tail.dim() == 3 and tail.shape[1:] == (max(taps - 1, 1), C) and tail.dtype == U.dtype,
+          "ssm_prepare: tail [slots, taps - 1, C] of the projection's dtype")
+    _need(all(t.dtype == torch.float32 and t.shape == (H,) for t in (a_log, dt_bias)),
+          "ssm_prepare: a_log, dt_bias float32 [H]")
+    dev = U.device
+    qn = torch.empty((T, G, N), dtype=torch.float32, device=dev)
+    kn = torch.empty((T, G, N), dtype=torch.float32, device=dev)
+    vv = torch.empty((T, H, dv), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    dec = torch.empty((T, H, 1), dtype=torch.float32, device=dev)
+    _check(_lib().illm_ssm_prepare(
+        _p(U), _code(U), U.shape[1], x_off, dt_off, _p(conv_w), _p(conv_b), taps, _p(tail), _p(row_slot),
+        _p(a_log), _p(dt_bias), _p(qn), _p(kn), _p(vv), _p(beta), _p(dec), T, G, H, N, dv,
+        1 if update_tail else 0, _stream()), "ssm_prepare")
+    return qn, kn, vv, beta, dec
+
+
+def ssm_finish(o: torch.Tensor, x: torch.Tensor, D: torch.Tensor, Z: torch.Tensor, z_off: int,
+               weight: torch.Tensor, norm_groups: int, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """[T, H dv] rows y = (o + D[h] x) silu(Z[:, z_off ..]), RMS-normed in `norm_groups` equal parts
+    of the row (each by its own root mean square), times weight [H dv]."""
+    _gpu(o, x, D, Z, weight)
+    T, H, dv = o.shape
+    _need(o.dtype == torch.float32 and x.dtype == torch.float32 and x.shape == o.shape
+          and D.dtype == torch.float32 and D.shape == (H,) and weight.shape == (H * dv,)
+          and Z.dim() == 2 and Z.shape[0] == T and Z.shape[1] >= z_off + H * dv
+          and norm_groups >= 1 and (H * dv) % norm_groups == 0, "ssm_finish: shapes")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    _check(_lib().illm_ssm_finish(_p(o), _p(x), _p(D), _p(Z), _code(Z), Z.shape[1], z_off, _p(weight),
+                                  _code(weight), _p(out), _code(out), T, H, dv, int(norm_groups),
+                                  ctypes.c_float(eps), _stream()), "ssm_finish")
+    return out
+
+
+def memory_prepare(U: torch.Tensor, i_off: int, f_off: int, i_bias: torch.Tensor, f_bias: torch.Tensor,
+                   cap: float, m_state: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+                   n_seqs: int, H: int, dk: int, dv: int):
+    """A matrix memory's float32 inputs for the plain gated rule, from U [T, n] = [q (H dk) | k (H dk)
+    | v (H dv) | ..]: q dk^-1/2, k, and v with a column of ones behind it (so the state's last
+    column sums the weighted keys); the gates i = cap tanh((U[:, i_off + h] + i_bias) / cap) and
+    f = logsigmoid(cap tanh((U[:, f_off + h] + f_bias) / cap)) against the running maximum
+    m_t = max(f + m_(t-1), i), token after token from `m_state` float32 [slots, H] and back into it:
+    decay exp(f + m_(t-1) - m_t), weight exp(i - m_t).
+    Returns (q [T, H, dk], k, v [T, H, dv + 1], weight [T, H], decay [T, H, 1], exp(-m) [T, H])."""
+    _gpu(U, i_bias, f_bias, m_state, cu_seqlens, seq_slot)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
+    T = U.shape[0]
+    _need(U.dim() == 2 and U.shape[1] >= max(2 * H * dk + H * dv, i_off + H, f_off + H),
+          "memory_prepare: projection too narrow")
+    _need(all(t.dtype == torch.float32 and t.shape == (H,) for t in (i_bias, f_bias))
+          and m_state.dtype == torch.float32 and m_state.dim() == 2 and m_state.shape[1] == H,
+          "memory_prepare: biases float32 [H], m_state float32 [slots, H]")
+    dev = U.device
+    qn = torch.empty((T, H, dk), dtype=torch.float32, device=dev)
+    kn = torch.empty((T, H, dk), dtype=torch.float32, device=dev)
+    vv = torch.empty((T, H, dv + 1), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    dec = torch.empty((T, H, 1), dtype=torch.float32, device=dev)
+    em = torch.empty((T, H), dtype=torch.float32, device=dev)
+    _check(_lib().illm_memory_prepare(
+        _p(U), _code(U), U.shape[1], i_off, f_off, _p(i_bias), _p(f_bias), ctypes.c_float(cap),
+        _p(m_state), _p(cu_seqlens), _p(seq_slot), _p(qn), _p(kn), _p(vv), _p(beta), _p(dec), _p(em), T,
+        n_seqs, H, dk, dv, _stream()), "memory_prepare")
+    return qn, kn, vv, beta, dec, em
+
+
+def memory_finish(o: torch.Tensor, em: torch.Tensor, weight: torch.Tensor, Z: torch.Tensor, z_off: int,
+                  eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """o float32 [T, H, dv + 1] (the last column n . q): y = o[..., :dv] / (max(|n . q|, em) + 1e-6),
+    then per head y / sqrt(mean y^2 + eps) * weight[h dv + j] * sigmoid(Z[:, z_off + h dv + j])."""
+    _gpu(o, em, weight, Z)
+    T, H, dv1 = o.shape
+    dv = dv1 - 1
+    _need(o.dtype == torch.float32 and em.dtype == torch.float32 and em.shape == (T, H)
+          and weight.shape == (H * dv,) and Z.dim() == 2 and Z.shape[0] == T
+          and Z.shape[1] >= z_off + H * dv, "memory_finish: shapes")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    _check(_lib().illm_memory_finish(_p(o), _p(em), _p(weight), _code(weight), _p(Z), _code(Z), Z.shape[1],
+                                     z_off, _p(out), _code(out), T, H, dv, ctypes.c_float(eps), _stream()),
+           "memory_finish")
+    return out
 
 
 DELTA_GATES = {"silu": 0, "sigmoid": 1}

@@ -1,3 +1,3 @@
-from . import kukupel, llama, rabapel  # registers Kukupel, LlamaForCausalLM and Rabapel
+from . import kukupel, llama, rabapel, sabipel  # registers Kukupel, LlamaForCausalLM, Rabapel and Sabipel
 
-__all__ = ["kukupel", "llama", "rabapel"]
+__all__ = ["kukupel", "llama", "rabapel", "sabipel"]

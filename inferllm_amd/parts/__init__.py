@@ -1,5 +1,5 @@
 from . import (attention, block, delta_rule, ends, feedforward, latent_attention, norm, position,  # registers
-               side_by_side)                                                                   # the built-in parts
+               recurrent, side_by_side)                                                                   # the built-in parts
 from .base import (Block, Embedding, FeedForward, Head, Mixer, Norm, Part, PositionEncoding,
                    StepContext, build_part, part_class, register_part)
 

@@ -224,3 +224,122 @@ class CappedAttention(Mixer):
                                     ctx.seq_slot, ctx.seq_len, nh, nkv, dk, dv, self.scale,
                                     self.softcap, window, nsplit)
         return ops.linear(o, self.w_o)
+
+
+@register_part("mixer", "gated_attention")
+class GatedAttention(Mixer):
+    """Causal softmax attention with grouped kv heads and key and value widths of their own, without
+    a rotation, put together from options:
+
+    * `qk_norm`: q and k each pass an RMS norm over the whole projection (all heads at once, before
+      they are split), with plain weights of that width and `eps`;
+    * `slope_power` p > 0: a bias by distance, score = q . k * scale - slope_h (i - j) with
+      slope_h = 2^(-p (h + 1) / H) for head h = 0 .. H - 1;
+    * `chunk` c > 0: position i sees j <= i only if floor(i / c) = floor(j / c), chunks counted from
+      the sequence's position 0; `window`: only the last `window` keys; `softcap` as in
+      `capped_attention` (applied before the bias);
+    * `value_mix` "source": the layer's values are handed on to later layers of the step;
+      "mixed": v <- (1 - lam) v + lam v_source with the stored scalar `value_mix` and the source
+      layer's values of the same token (the mixed v is what the cache keeps);
+    * `gate`: the heads' outputs side by side times sigmoid(W_g h) before the output projection.
+
+    Scores, softmax, norms and the mixing are float32.  A step stores its keys and values in the
+    paged cache first and every row attends over the cache at its position, so prompts, portions
+    of prompts and single tokens run the same way.
+    """
+
+    graph_safe_prompts = True
+    takes_continuations = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
+                 value_dim: int, softmax_scale: Optional[float] = None, softcap: float = 0.0,
+                 window: Optional[int] = None, chunk: int = 0, slope_power: float = 0.0,
+                 qk_norm: bool = False, eps: float = 1e-6, value_mix: Optional[str] = None,
+                 gate: bool = False, tensors=None):
+        super().__init__(tensors)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if key_dim > 256 or value_dim > 256:
+            raise ValueError(f"head sizes {key_dim}, {value_dim} are beyond the attention kernels' limit of 256")
+        if value_mix not in (None, "source", "mixed"):
+            raise ValueError(f"value_mix {value_mix!r}: None, 'source' or 'mixed'")
+        self.E, self.nh, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dk, self.dv = int(key_dim), int(value_dim)
+        self.window = int(window) if window else None
+        self.chunk = int(chunk or 0)
+        self.scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(self.dk)
+        self.softcap, self.slope_power = float(softcap or 0.0), float(slope_power or 0.0)
+        self.qk_norm, self.eps, self.value_mix, self.gate = bool(qk_norm), float(eps), value_mix, bool(gate)
+        self.k_off = self.nh * self.dk
+        self.v_off = self.k_off + self.nkv * self.dk
+        self.g_off = self.v_off + self.nkv * self.dv
+        self.slopes = self.lam = self.q_norm = self.k_norm = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        keep = dict(keep_stored=True)
+        out = {"q": TensorWant((self.nh * self.dk, self.E)), "k": TensorWant((self.nkv * self.dk, self.E)),
+               "v": TensorWant((self.nkv * self.dv, self.E)), "o": TensorWant((self.E, self.nh * self.dv))}
+        if self.qk_norm:
+            out["q_norm"] = TensorWant((self.nh * self.dk,), init="ones_normal", **keep)
+            out["k_norm"] = TensorWant((self.nkv * self.dk,), init="ones_normal", **keep)
+        if self.value_mix == "mixed":
+            out["value_mix"] = TensorWant((), **keep)
+        if self.gate:
+            out["g"] = TensorWant((self.nh * self.dv, self.E))
+        return out
+
+    def kv_spec(self) -> KVSpec:
+        from ..cache.manager import TokenTensor
+        return KVSpec("window" if self.window else "full",
+                      (TokenTensor("k", (self.nkv, self.dk)), TokenTensor("v", (self.nkv, self.dv))),
+                      self.window)
+
+    def load(self, tensors) -> None:
+        take = lambda n: self._take(tensors, n)
+        rows = [take(n) for n in ("q", "k", "v")] + ([take("g")] if self.gate else [])
+        self.w_in = ops.decode_weight(_fuse(rows), "plain", self.decode_copies)     # [q | k | v | g]
+        self.w_o = ops.decode_weight(take("o").contiguous(), "plain", self.decode_copies)
+        dev = take("q").device
+        if self.qk_norm:
+            self.q_norm, self.k_norm = take("q_norm").contiguous(), take("k_norm").contiguous()
+        if self.value_mix == "mixed":
+            self.lam = take("value_mix").to(torch.float32).reshape(1).contiguous()
+        if self.slope_power > 0:
+            h = torch.arange(1, self.nh + 1, dtype=torch.float64)
+            self.slopes = torch.pow(2.0, -self.slope_power * h / self.nh).to(torch.float32).to(dev)
+
+    def tunables(self):
+        return (("plain", self.w_o, {}),)
+
+    def forward(self, h, ctx: StepContext, line, writes_cache, position):
+        nh, nkv, dk, dv = self.nh, self.nkv, self.dk, self.dv
+        kc, vc, group = ctx.cache.kv_line(line)
+        window = self.window or 0
+        rows = ops.linear(h, self.w_in)
+        first, first_off = None, 0
+        if self.value_mix == "mixed":
+            first, first_off, width = ctx.exchange["value_mix_source"]
+            if width != nkv * dv:
+                raise ValueError(f"value mixing: the source layer's values are {width} wide, this layer's {nkv * dv}")
+        store = writes_cache
+        ops.qkv_norm_mix_store(rows, self.k_off, self.v_off, self.q_norm, self.k_norm, self.eps,
+                               self.lam if first is not None else None, first, first_off, ctx.row_pos,
+                               ctx.row_slot, kc if store else None, vc if store else None, group.table,
+                               group.page_size, group.ring, nh, nkv, dk, dv)
+        if self.value_mix == "source":
+            ctx.exchange["value_mix_source"] = (rows, self.v_off, nkv * dv)
+        gate = rows if self.gate else None
+        if ctx.prefill:
+            o = ops.attn_cap_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, group.table,
+                                  group.page_size, group.ring, ctx.n_seqs, ctx.max_rows, nh, nkv, dk, dv,
+                                  self.scale, self.softcap, window, self.slopes, self.chunk, gate, self.g_off)
+        else:
+            longest = ctx.max_len
+            for bound in (window, self.chunk):
+                longest = min(longest, bound) if bound else longest
+            tiles = max(1, (longest + 63) // 64)
+            nsplit = max(1, min(-(-512 // max(1, ctx.n_seqs * nh)), 16, tiles))
+            o = ops.attn_cap_decode(rows, kc, vc, group.table, group.page_size, group.ring, ctx.seq_slot,
+                                    ctx.seq_len, nh, nkv, dk, dv, self.scale, self.softcap, window,
+                                    nsplit, self.slopes, self.chunk, gate, self.g_off)
+        return ops.linear(o, self.w_o)

@@ -52,6 +52,8 @@ class PreNormBlock(Block):
 @register_part("block", "parallel")
 class ParallelBlock(Block):
     """x <- x + (mixer(h) + feed_forward(h)) with h = norm(x): one norm, both parts read its rows.
+    With a second norm (`feed_forward_norm`) the feed-forward reads rows of its own,
+    x <- x + (mixer(norm1(x)) + feed_forward(norm2(x))), both norms of the same x.
 
     The two outputs are left for the next norm to add to the stream as (mixer + feed-forward) in
     float32: as a pair, if that norm says it adds pairs in its own kernel (`Norm.adds_pairs`), else
@@ -71,7 +73,9 @@ class ParallelBlock(Block):
             pending = ops.sum_rows(*pending)
         h = self.mixer_norm.forward(x, pending, ctx)
         a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
-        f = self.feed_forward.forward(h, ctx)
+        # a second norm reads the same x, which holds the sum by now
+        two = self.feed_forward_norm is not None
+        f = self.feed_forward.forward(self.feed_forward_norm.forward(x, None, ctx) if two else h, ctx)
         if f is None:
             return a
         if next_norm is not None and getattr(next_norm, "adds_pairs", False):

@@ -5,6 +5,7 @@ from typing import Dict, Optional
 
 import torch
 
+from ..cache.manager import StateSpec
 from ..kernels import ops
 from ..weights.loader import TensorWant
 from .base import Embedding, Head, StepContext, register_part
@@ -35,6 +36,58 @@ class TokenEmbedding(Embedding):
         if self.streams:
             return ops.embed(ctx.tokens, self.weight, self.scale, self.streams)
         return ops.embed(ctx.tokens, self.weight, self.scale)
+
+
+@register_part("embedding", "token_pair_embedding")
+class TokenPairEmbedding(Embedding):
+    """The token's row times `scale`, plus a row of a table hashed by the pair (previous token, token),
+    plus a learned row of the position:
+
+        x = table[t] * scale + pairs[(t_before * mul_prev + t * mul_cur) mod buckets] + places[p]
+
+    A sequence's first token takes the pair table's last row (number `buckets`).  The token before
+    a step's first row is part of the sequence's state: one int per slot, kept by the cache manager
+    under the line `STATE_LINE` like a mixer's state.  `buckets` 0: no pair table; `positions` 0: no
+    position table.  All sums are float32."""
+
+    graph_safe_prompts = True
+    STATE_LINE = "embedding"
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, buckets: int = 0,
+                 mul_prev: int = 1, mul_cur: int = 1, positions: int = 0, tensors=None):
+        super().__init__(tensors)
+        self.V, self.E, self.scale = int(vocab_size), int(hidden_size), float(scale)
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.positions = int(positions)
+        if self.buckets < 0 or self.mul_prev < 0 or self.mul_cur < 0 or self.positions < 0:
+            raise ValueError("token_pair_embedding: buckets, multipliers and positions are not negative")
+        self.weight = self.pairs = self.places = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        out = {"weight": TensorWant((self.V, self.E))}
+        if self.buckets:
+            out["pairs"] = TensorWant((self.buckets + 1, self.E))
+        if self.positions:
+            out["places"] = TensorWant((self.positions, self.E))
+        return out
+
+    def state_spec(self):
+        """The last token of every sequence (int32), if there is a pair table."""
+        return StateSpec((), torch.int32) if self.buckets else None
+
+    def load(self, tensors) -> None:
+        self.weight = self._take(tensors, "weight").contiguous()
+        self.pairs = self._take(tensors, "pairs").contiguous() if self.buckets else None
+        self.places = self._take(tensors, "places").contiguous() if self.positions else None
+
+    def forward(self, ctx: StepContext):
+        last = ctx.cache.state_line(self.STATE_LINE) if self.buckets else None
+        x = ops.embed_pairs(ctx.tokens, ctx.row_pos, ctx.row_slot, self.weight, self.scale, self.pairs,
+                            self.buckets, self.mul_prev, self.mul_cur, self.places, last,
+                            remember=not ctx.prefill)
+        if ctx.prefill and last is not None:
+            ops.remember_last(ctx.tokens, ctx.cu_seqlens, ctx.seq_slot, last, ctx.n_seqs)
+        return x
 
 
 @register_part("head", "lm_head")

@@ -69,12 +69,14 @@ class NoFeedForward(FeedForward):
         return None
 
 
-_ACTIVATIONS = {"relu_squared": "relu_squared"}        # activation -> the op that computes it
+# activation -> the op that computes it
+_ACTIVATIONS = {"relu_squared": "relu_squared", "gelu_tanh": "gelu_tanh"}
 
 
 @register_part("feed_forward", "dense_activation")
 class DenseActivation(FeedForward):
-    """down(act(up h)) without a gate; `activation` "relu_squared": max(z, 0)^2."""
+    """down(act(up h)) without a gate; `activation` "relu_squared": max(z, 0)^2, or "gelu_tanh":
+    0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
 
     graph_safe_prompts = True
 

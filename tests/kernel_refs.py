@@ -440,16 +440,45 @@ def kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table,
         vcache[page, :, at, :] = rows[r, v_off:v_off + nkv * dv].view(nkv, dv)
 
 
-def _attend_capped(q, k, v, scale, cap):
-    """q [nh, dk], k [L, nkv, dk], v [L, nkv, dv]: every key visible."""
-    nh, per = q.shape[0], q.shape[0] // k.shape[1]
+def _attend_capped(q, k, v, scale, cap, slopes=None):
+    """q [nh, dk], k [L, nkv, dk], v [L, nkv, dv]: every key visible, the last one the query's own."""
+    nh, per, L = q.shape[0], q.shape[0] // k.shape[1], k.shape[0]
     out = torch.zeros(nh, v.shape[2], dtype=F64)
     for h in range(nh):
         s = (k[:, h // per, :].to(F64) @ q[h].to(F64)) * scale
         if cap:
             s = cap * torch.tanh(s / cap)
+        if slopes is not None:
+            s = s - slopes[h].to(F64) * torch.arange(L - 1, -1, -1, dtype=F64)
         out[h] = torch.softmax(s, dim=0) @ v[:, h // per, :].to(F64)
     return out
+
+
+def _first_seen(pos, window, chunk):
+    first = max(0, pos - window + 1) if window and window > 0 else 0
+    return max(first, pos // chunk * chunk) if chunk and chunk > 0 else first
+
+
+def _gated(out_row, gate, r, gate_off):
+    if gate is None:
+        return out_row
+    return out_row * torch.sigmoid(gate[r, gate_off:gate_off + out_row.numel()].to(F64))
+
+
+def qkv_norm_mix_store(rows, k_off, v_off, q_weight, k_weight, eps, lam, first, first_off, row_pos, row_slot,
+                       kcache, vcache, page_table, page_size, ring, nh, nkv, dk, dv):
+    def normed(x, w):
+        x = x.to(F64)
+        return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.to(F64)).to(rows.dtype)
+    if q_weight is not None:
+        rows[:, :nh * dk] = normed(rows[:, :nh * dk], q_weight)
+        rows[:, k_off:k_off + nkv * dk] = normed(rows[:, k_off:k_off + nkv * dk], k_weight)
+    if lam is not None:
+        l = lam.to(F64)[0]
+        rows[:, v_off:v_off + nkv * dv] = ((1 - l) * rows[:, v_off:v_off + nkv * dv].to(F64)
+                                           + l * first[:, first_off:first_off + nkv * dv].to(F64)).to(rows.dtype)
+    if kcache is not None:
+        kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table, page_size, ring, nkv, dk, dv)
 
 
 def _cached(kcache, vcache, page_table, slot, first, total, page_size, ring):
@@ -458,26 +487,29 @@ def _cached(kcache, vcache, page_table, slot, first, total, page_size, ring):
 
 
 def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, page_size, ring,
-                  n_seqs, max_rows, nh, nkv, dk, dv, scale, cap, window):
+                  n_seqs, max_rows, nh, nkv, dk, dv, scale, cap, window, slopes=None, chunk=0, gate=None,
+                  gate_off=0):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(n_seqs):
         s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
         for a in range(s1 - s0):
             pos = int(seq_start[b]) + a
-            first = max(0, pos - window + 1) if window and window > 0 else 0
+            first = _first_seen(pos, window, chunk)
             k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, pos + 1, page_size, ring)
-            out[s0 + a] = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap).reshape(-1).to(q.dtype)
+            row = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
+            out[s0 + a] = _gated(row, gate, s0 + a, gate_off).to(q.dtype)
     return out
 
 
 def attn_cap_decode(q, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, dk, dv,
-                    scale, cap, window, nsplit):
+                    scale, cap, window, nsplit, slopes=None, chunk=0, gate=None, gate_off=0):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(q.shape[0]):
         n = int(seq_len[b])
-        first = max(0, n - window) if window and window > 0 else 0
+        first = _first_seen(n - 1, window, chunk)
         k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, n, page_size, ring)
-        out[b] = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap).reshape(-1).to(q.dtype)
+        row = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
+        out[b] = _gated(row, gate, b, gate_off).to(q.dtype)
     return out
 
 
@@ -511,8 +543,9 @@ def delta_prepare(P, b_off, A, a_off, conv_w, tail, row_slot, a_log, dt_bias, G,
     return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, beta, dec))
 
 
-def delta_conv_tail(P, tail, cu_seqlens, seq_slot, n_seqs, taps):
+def delta_conv_tail(P, tail, cu_seqlens, seq_slot, n_seqs, taps, col_off=0):
     K, C = taps - 1, tail.shape[2]
+    P = P[:, col_off:]
     for b in range(n_seqs if K else 0):
         r0, n, slot = int(cu_seqlens[b]), int(cu_seqlens[b + 1]) - int(cu_seqlens[b]), int(seq_slot[b])
         if n <= 0:
@@ -523,7 +556,7 @@ def delta_conv_tail(P, tail, cu_seqlens, seq_slot, n_seqs, taps):
             tail[slot, j] = P[r0 + at, :C].to(tail.dtype) if at >= 0 else old[j + n]
 
 
-def delta_scan(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot, n_seqs, max_rows):
+def delta_scan(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot, n_seqs, max_rows, correct=True):
     T, G, dk = qn.shape
     H, dv = vv.shape[1], vv.shape[2]
     o = torch.zeros(T, H, dv, dtype=torch.float32)
@@ -533,7 +566,7 @@ def delta_scan(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot, n_seqs, max_r
             for h in range(H):
                 g = h // (H // G)
                 S = state[slot, h].to(F64) * dec[r, h].to(F64).expand(dk)[:, None]
-                u = beta[r, h].to(F64) * (vv[r, h].to(F64) - S.t() @ kn[r, g].to(F64))
+                u = beta[r, h].to(F64) * (vv[r, h].to(F64) - (S.t() @ kn[r, g].to(F64) if correct else 0.0))
                 S = S + torch.outer(kn[r, g].to(F64), u)
                 o[r, h] = (S.t() @ qn[r, g].to(F64)).to(torch.float32)
                 state[slot, h] = S.to(torch.float32)
@@ -548,6 +581,108 @@ def delta_finish(o, weight, Z, z_off, gate, eps, out_dtype):
     return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(F64) * act).reshape(T, H * dv).to(out_dtype)
 
 
+# ---------------------------------------------------------------- around the plain gated rule
+def _softplus(a):
+    return torch.where(a > 30, a, torch.log1p(torch.exp(torch.clamp(a, max=30))))
+
+
+def ssm_prepare(U, x_off, dt_off, conv_w, conv_b, tail, row_slot, a_log, dt_bias, G, H, N, dv, update_tail=False):
+    T, C, taps = U.shape[0], conv_w.shape[0], conv_w.shape[1]
+    K, inner, GN = taps - 1, H * dv, G * N
+    X = U[:, x_off:x_off + C]
+    y = conv_b.to(F64).expand(T, C).clone()
+    for r in range(T):
+        slot, before = int(row_slot[r]), 0
+        while before < K and r - before - 1 >= 0 and int(row_slot[r - before - 1]) == slot:
+            before += 1
+        for j in range(taps):
+            d = K - j
+            src = X[r - d] if d <= before else tail[slot, K - (d - before)]
+            y[r] += conv_w[:, j].to(F64) * src.to(F64)
+    y = y * torch.sigmoid(y)
+    vv, kn, qn = y[:, :inner].view(T, H, dv), y[:, inner:inner + GN].view(T, G, N), y[:, inner + GN:].view(T, G, N)
+    step = _softplus(U[:, dt_off:dt_off + H].to(F64) + dt_bias.to(F64))
+    dec = torch.exp(-torch.exp(a_log.to(F64)) * step).view(T, H, 1)
+    if update_tail:
+        for r in range(T if K else 0):
+            slot = int(row_slot[r])
+            tail[slot] = torch.cat([tail[slot, 1:], X[r:r + 1].to(tail.dtype)])
+    return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, step, dec))
+
+
+def ssm_finish(o, x, D, Z, z_off, weight, norm_groups, eps, out_dtype):
+    T, H, dv = o.shape
+    z = Z[:, z_off:z_off + H * dv].to(F64)
+    y = (o.to(F64) + D.to(F64)[None, :, None] * x.to(F64)).reshape(T, H * dv) * (z * torch.sigmoid(z))
+    y = y.view(T, norm_groups, -1)
+    y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, H * dv) * weight.to(F64)).to(out_dtype)
+
+
+def memory_prepare(U, i_off, f_off, i_bias, f_bias, cap, m_state, cu_seqlens, seq_slot, n_seqs, H, dk, dv):
+    T = U.shape[0]
+    qn = U[:, :H * dk].to(F64).view(T, H, dk) * dk ** -0.5
+    kn = U[:, H * dk:2 * H * dk].to(F64).view(T, H, dk)
+    vv = torch.cat([U[:, 2 * H * dk:2 * H * dk + H * dv].to(F64).view(T, H, dv), torch.ones(T, H, 1, dtype=F64)], dim=2)
+    ig = cap * torch.tanh((U[:, i_off:i_off + H].to(F64) + i_bias.to(F64)) / cap)
+    fg = -_softplus(-(cap * torch.tanh((U[:, f_off:f_off + H].to(F64) + f_bias.to(F64)) / cap)))
+    beta, dec, em = (torch.zeros(T, H, dtype=F64) for _ in range(3))
+    for b in range(n_seqs):
+        slot = int(seq_slot[b])
+        m = m_state[slot].to(F64)
+        for r in range(int(cu_seqlens[b]), int(cu_seqlens[b + 1])):
+            new = torch.maximum(fg[r] + m, ig[r])
+            dec[r], beta[r], em[r] = torch.exp(fg[r] + m - new), torch.exp(ig[r] - new), torch.exp(-new)
+            m = new
+        if int(cu_seqlens[b + 1]) > int(cu_seqlens[b]):
+            m_state[slot] = m.to(torch.float32)
+    return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, beta, dec.view(T, H, 1), em))
+
+
+def memory_finish(o, em, weight, Z, z_off, eps, out_dtype):
+    T, H, dv1 = o.shape
+    dv = dv1 - 1
+    x = o.to(F64)
+    den = torch.maximum(x[:, :, dv].abs(), em.to(F64)) + 1e-6
+    y = x[:, :, :dv] / den[:, :, None]
+    y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps)
+    z = Z[:, z_off:z_off + H * dv].to(F64)
+    return (y.reshape(T, H * dv) * weight.to(F64) * torch.sigmoid(z)).to(out_dtype)
+
+
+def embed_pairs(tokens, row_pos, row_slot, table, scale, pairs, buckets, mul_prev, mul_cur, places, last_token,
+                remember):
+    T = tokens.numel()
+    out = torch.zeros(T, table.shape[1], dtype=torch.float32)
+    for t in range(T):
+        tok, pos, slot = int(tokens[t]), int(row_pos[t]), int(row_slot[t])
+        v = table[tok].to(F64) * scale
+        if pairs is not None:
+            if pos == 0:
+                at = buckets
+            else:
+                prev = int(tokens[t - 1]) if t > 0 and int(row_slot[t - 1]) == slot else int(last_token[slot])
+                at = (prev * mul_prev + tok * mul_cur) % buckets
+            v = v + pairs[at].to(F64)
+        if places is not None:
+            v = v + places[pos].to(F64)
+        out[t] = v.to(torch.float32)
+        if remember and last_token is not None:
+            last_token[slot] = tok
+    return out
+
+
+def remember_last(tokens, cu_seqlens, seq_slot, last_token, n_seqs):
+    for b in range(n_seqs):
+        if int(cu_seqlens[b + 1]) > int(cu_seqlens[b]):
+            last_token[int(seq_slot[b])] = int(tokens[int(cu_seqlens[b + 1]) - 1])
+
+
+def gelu_tanh(x):
+    z = x.to(F64)
+    return (0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))).to(x.dtype)
+
+
 def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
@@ -559,6 +694,7 @@ def patch(monkeypatch):
                  "latent_store_absorb",
                  "few_outputs_f32", "moe_route", "moe_plan", "moe_experts", "moe_combine",
                  "stream_mix_norm", "kv_store2", "attn_cap_rows", "attn_cap_decode", "delta_prepare",
-                 "delta_conv_tail", "delta_scan", "delta_finish"):
+                 "delta_conv_tail", "delta_scan", "delta_finish", "qkv_norm_mix_store", "ssm_prepare",
+                 "ssm_finish", "memory_prepare", "memory_finish", "embed_pairs", "remember_last", "gelu_tanh"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(ops.ScaledSum, "tensor", scaled_sum_tensor)
