@@ -103,8 +103,10 @@ def mlstm(h, w, p, m, eps):
     return o @ w[p + "o"].T
 
 
-def attention(h, w, p, m, eps, first_values, is_first):
-    """Returns (output, the values this layer would hand on as the first layer's)."""
+def attention(h, w, p, m, eps, first_values, is_first, edge_shift=0):
+    """Returns (output, the values this layer would hand on as the first layer's).  `edge_shift`
+    moves every chunk's first visible key by that many positions: what an implementation that is
+    off by one at the edge would compute (for tests that show a fault there would be seen)."""
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     T, rep = h.shape[0], m["heads"] // m["kv_heads"]
     q = rms_norm(h @ w[p + "q"].T, w[p + "q.norm"], eps).view(T, H, dk)
@@ -120,6 +122,7 @@ def attention(h, w, p, m, eps, first_values, is_first):
     j = torch.arange(T)
     for i in range(T):
         lo = (i // chunk) * chunk if chunk else 0
+        lo = min(max(lo + edge_shift, 0), i)
         for hh in range(H):
             slope = 2.0 ** (-8.0 * (hh + 1) / H)
             s = (k[lo:i + 1, hh // rep] @ q[i, hh]) * m["scale"] - slope * (i - j[lo:i + 1])
@@ -132,7 +135,7 @@ def dense(h, w, p):
     return gelu_tanh(h @ w[p + "up"].T) @ w[p + "down"].T
 
 
-def forward(config, w, ids, layers_out=None):
+def forward(config, w, ids, layers_out=None, edge_shift=0):
     """float64 logits [T, vocab] of one sequence from its first token on."""
     eps = config["norm"]["eps"]
     x = embed(w, config["embedding"], ids)
@@ -146,7 +149,7 @@ def forward(config, w, ids, layers_out=None):
             a = mlstm(h, w, p, m, eps)
         else:
             is_first = bool(m.get("v_mix")) and first_values is None
-            a, handed = attention(h, w, p, m, eps, first_values, is_first)
+            a, handed = attention(h, w, p, m, eps, first_values, is_first, edge_shift)
             if is_first:
                 first_values = handed
         if layer.get("mlp") is not None:
