@@ -22,11 +22,13 @@ of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
 The run fails (non-zero) if any timed run produced a non-finite logit or the same
 greedy token everywhere.
 
-`--design rabapel` and `--design kukupel` are other workloads with a line of their own (the
+`--design rabapel`, `--design kukupel` and `--design sabipel` are other workloads with a line of their own (the
 default's stays as it is):
 Rabapel (latent attention, layers that alternate a dense and a routed feed-forward) at two
 sizes beside LLaMA at the same width, heads and layer count: prefill of 2,048 tokens and decoding
 at batch 1, 8 and 64, each with its fraction of the matrix or HBM peak.
+Kukupel likewise beside Rabapel, and Sabipel (state-space, matrix-memory and chunked-attention
+layers with dense feed-forwards) beside Kukupel.
 """
 import argparse
 import json
@@ -424,6 +426,107 @@ def kukupel_main(args) -> int:
     return 0
 
 
+def sabipel_config(width, heads, kv_heads, layers, chunk=1024, vocab=32000):
+    """Layers in the order mamba2, attention, mlstm, attention ...: state-space heads of 64 value
+    dims on a state of 128 (an inner width of twice the model's), matrix-memory heads of 128 x 128,
+    attention heads of 128 query and 128 value dims in chunks of `chunk` positions, a dense
+    feed-forward of four times the width in every layer."""
+    ssm = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+    mem = {"heads": heads, "dim": 128, "vdim": 128, "gate_cap": 15.0}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+           "mask": {"size": chunk}, "v_mix": True}
+    mlp = {"kind": "dense", "ff": 4 * width}
+    kinds = [("mamba2", ssm), ("attention", att), ("mlstm", mem), ("attention", att)]
+    return {"architecture": "Sabipel", "vocab": vocab, "width": width, "max_positions": 8192,
+            "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "layers": [{"type": kinds[i % 4][0], "mixer": dict(kinds[i % 4][1]), "mlp": dict(mlp)}
+                       for i in range(layers)]}
+
+
+def sabipel_counts(cfg, esz):
+    """(step_bytes(batch, mean_ctx), flops(tokens, lens)) of a Sabipel configuration: the weights a
+    decode step reads, attention's cache rows within a chunk, the recurrent layers' float32 states
+    (read and written); the multiply-adds of a prompt step (attention within its chunks, the
+    recurrence as 2 key x value products a token and head)."""
+    E, V = cfg["width"], cfg["vocab"]
+
+    def layer_parts(layer):
+        """(weights, float32 state, cache columns a token, score columns a pair, chunk)"""
+        m, kind = layer["mixer"], layer["type"]
+        ff = 2 * E * layer["mlp"]["ff"] if layer.get("mlp") else 0
+        if kind == "mamba2":
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            return E * (2 * inner + 2 * gn + m["heads"]) + inner * E + ff, m["heads"] * m["state"] * m["vdim"], 0, 0, 0
+        if kind == "mlstm":
+            H, dk, dv = m["heads"], m["dim"], m["vdim"]
+            return E * (2 * H * dk + 2 * H * dv + 2 * H) + H * dv * E + ff, H * dk * (dv + 1), 0, 0, 0
+        H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        return (E * (H * dk + G * dk + G * dv + H * dv) + H * dv * E + ff, 0, G * (dk + dv), H * (dk + dv),
+                (m.get("mask") or {}).get("size", 0))
+
+    def seen(n, chunk):
+        """keys that position n - 1 sees"""
+        return (n - 1) % chunk + 1 if chunk else n
+
+    def step_bytes(batch, mean_ctx):
+        total = V * E * esz + batch * 3 * E * esz
+        for layer in cfg["layers"]:
+            w, state, kv_row, _, chunk = layer_parts(layer)
+            total += (w + batch * seen(int(mean_ctx), chunk) * kv_row) * esz + batch * state * 4 * 2
+        return total
+
+    def flops(tokens, lens):
+        total = 2.0 * len(lens) * V * E
+        for layer in cfg["layers"]:
+            w, state, _, qk, chunk = layer_parts(layer)
+            pairs = sum(sum(seen(p + 1, chunk) for p in range(n)) for n in lens) if qk else 0
+            total += 2.0 * tokens * w + 2.0 * qk * pairs + 2.0 * 2 * state * tokens
+        return total
+
+    return step_bytes, flops
+
+
+def sabipel_main(args) -> int:
+    """Sabipel at two sizes beside Kukupel, the library's other design with recurrent layers that
+    keep a matrix of state per head, at the same width, heads and number of layers (four): tokens/s
+    of these four-layer models, with the fraction of the matrix peak for prompts and of the HBM peak
+    for decode steps."""
+    import torch
+    from inferllm_amd import Engine
+    layers = args.layers or 4
+    esz = 2 if args.dtype == "bfloat16" else 4
+    sizes = {"2048": dict(width=2048, heads=16, kv_heads=4), "4096": dict(width=4096, heads=32, kv_heads=8)}
+    experts = {"2048": dict(experts=64, expert_ff=1408, top=6), "4096": dict(experts=32, expert_ff=2048, top=4)}
+    few = min(args.steps, 128)
+    out = {"metric": "Sabipel beside Kukupel at equal width, heads and layers: prefill tok/s at 2,048 tokens, decode tok/s at batch 1/8/64",
+           "unit": "tokens/s", "n_gpus": 1, "steps": few, "warmup": 4, "dtype": "bf16" if esz == 2 else "fp32",
+           "data": "synthetic: seeded random weights, uniform random token ids", "layers": layers, "sizes": {}}
+    for name, sz in sizes.items():
+        if args.size and args.size != name:
+            continue
+        row = {}
+        scfg = sabipel_config(layers=layers, **sz)
+        kcfg = kukupel_config(layers=layers, **sz, **experts[name])
+        for design, cfg, counts in (("sabipel", scfg, sabipel_counts), ("kukupel", kcfg, kukupel_counts)):
+            if args.only and args.only != design:
+                continue
+            eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, device="cuda:0", max_batch=64,
+                                     max_seq_len=4096, max_tokens=64 * 1024)
+            b = Bench.around(eng, cfg["vocab"], layers, args.dtype, *counts(cfg, esz))
+            torch.cuda.synchronize()
+            r = {"prefill_2048": b.prefill_run(2048, reps=4)}
+            if not args.prefill_only:
+                for batch in (1, 8, 64):
+                    v, ms, f = b.decode_run(batch, few, 4, args.prompt)
+                    r[f"decode_b{batch}"] = {"value": round(v, 1), "ms": round(ms, 4), "hbm_frac": round(f, 4)}
+            row[design] = r
+            b.close()
+            del b, eng
+        out["sizes"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -441,11 +544,12 @@ def main() -> int:
     ap.add_argument("--no-70b", action="store_true",
                     help="leave the LLaMA-2-70B shape out of `points` (138 GB of weights: half a minute)")
     ap.add_argument("--with-70b", action="store_true", help="(the default now; kept for old command lines)")
-    ap.add_argument("--design", default="llama", choices=["llama", "rabapel", "kukupel"],
+    ap.add_argument("--design", default="llama", choices=["llama", "rabapel", "kukupel", "sabipel"],
                     help="rabapel: that design at two sizes beside LLaMA at equal size (a line of its own); "
-                         "kukupel: that design at two sizes beside Rabapel at equal size (likewise)")
-    ap.add_argument("--size", default="", help="with --design rabapel or kukupel: only this width (2048 or 4096)")
-    ap.add_argument("--only", default="", help="with --design kukupel: only this one of the two designs")
+                         "kukupel: that design at two sizes beside Rabapel at equal size (likewise); "
+                         "sabipel: that design at two sizes beside Kukupel at equal size (likewise)")
+    ap.add_argument("--size", default="", help="with --design rabapel, kukupel or sabipel: only this width (2048 or 4096)")
+    ap.add_argument("--only", default="", help="with --design kukupel or sabipel: only this one of the two designs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
@@ -455,6 +559,8 @@ def main() -> int:
         return rabapel_main(args)
     if args.design == "kukupel":
         return kukupel_main(args)
+    if args.design == "sabipel":
+        return sabipel_main(args)
 
     shape_name, shape_cfg = SHAPES[args.shape]
     ctx_len = shape_cfg["max_position_embeddings"]

@@ -42,6 +42,10 @@ void illm_set_rows_shape(int tb, int kp);
 // csrc/gemm_rows.hip: rows of X a launch of its products takes, 64 or 128 (default).
 void illm_set_rows_a_launch(int rows);
 
+// illm_attn_cap_rows: 0 sends every size to the kernel on the vector units, which sizes beyond 128
+// or not in steps of 4 use, instead of the one on the matrix cores' float32 instruction (default 1).
+void illm_set_attn_cap_mfma(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -255,6 +255,190 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
     }
 }
 
+// ---------------------------------------------------------------- the same rows on the matrix cores
+// Key and value widths of up to 128 in steps of 4: both products on the float32 instruction of the
+// matrix cores (MFMA 32x32x2: float32 operands, products and sums), so scores and weights stay
+// float32 whatever the storage.  grid (tiles of 128 queries, heaviest first; heads; sequences); a
+// wave takes 32 queries.  Both products are kept transposed so that a lane's column is its query:
+// scores^T = K . Q^T puts the 16 scores of query (lane % 32) into a lane and its partner 32 lanes on
+// (max and sum: one exchange), and in context^T = V^T . P^T the lane's own 16 weights are the second
+// operand as they stand.  Keys and values go through LDS 32 keys at a time as float32, widths filled
+// up with zeros to whole tiles of 32 (KT, VT); the next tile's loads are in flight while this one is
+// multiplied.  A wave leaves out tiles that none of its rows sees (after them, before their window or
+// before their chunk).
+typedef float cap_f32x16_t __attribute__((ext_vector_type(16)));
+#define MQ 128  // query rows of a block
+#define MK 32   // keys of a tile
+
+template <int DT>
+__device__ __forceinline__ void ld4(const void* p, size_t at, float* x) {
+    if (DT == ILLM_BF16) {
+        const uint2 r = *(const uint2*)((const bf16_t*)p + at);
+        x[0] = __uint_as_float(r.x << 16); x[1] = __uint_as_float(r.x & 0xffff0000u);
+        x[2] = __uint_as_float(r.y << 16); x[3] = __uint_as_float(r.y & 0xffff0000u);
+    } else {
+        const float4 r = *(const float4*)((const float*)p + at);
+        x[0] = r.x; x[1] = r.y; x[2] = r.z; x[3] = r.w;
+    }
+}
+
+template <int DT, int KT, int VT>
+__global__ void __launch_bounds__(256, 2)
+attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __restrict__ out,
+                          const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot,
+                          const int32_t* __restrict__ seq_start, const void* __restrict__ kcache,
+                          const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
+                          int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
+                          float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
+                          const void* __restrict__ gate, int gate_stride, int gate_off) {
+    constexpr int DKP = 32 * KT, DVP = 32 * VT, KLD = DKP + 1;
+    __shared__ float ks[MK * KLD];
+    __shared__ float vs[MK * DVP];
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * MQ;
+    if (q0 >= len) return;
+    const int pos0 = seq_start[b], slot = seq_slot[b];
+    const int total = pos0 + len;
+    const int kvh = h / (nh / nkv);
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+    const int col = lane & 31, half = lane >> 5;
+    const int qrow = q0 + 32 * wave + col;                 // row within the step's rows of the sequence
+    const int qpos = pos0 + qrow;
+    const bool wave_has_rows = q0 + 32 * wave < len;
+    const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+    const float slope = slopes ? slopes[h] : 0.f;
+
+    // the query row: dims 2 s + half (zeros beyond dk)
+    float qr[DKP / 2];
+    {
+        const size_t at = (size_t)(start + min(qrow, len - 1)) * q_stride + (size_t)h * dk;
+#pragma unroll
+        for (int j = 0; j < DKP / 4; ++j) {
+            float x[4] = {0.f, 0.f, 0.f, 0.f};
+            if (4 * j < dk) ld4<DT>(q, at + 4 * j, x);
+            qr[2 * j] = half ? x[1] : x[0];
+            qr[2 * j + 1] = half ? x[3] : x[2];
+        }
+    }
+    // a thread's share of a tile: quads e = tid + 256 i of [32 keys][DKP / 4] and of [32 keys][DVP / 4]
+    float kreg[KT][4], vreg[VT][4];
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KT; ++i) {
+            const int e = tid + 256 * i, row = e / (DKP / 4), d = 4 * (e % (DKP / 4));
+            const int kj = min(k0 + row, total - 1);       // keys past the end: a valid row, masked below
+            kreg[i][0] = kreg[i][1] = kreg[i][2] = kreg[i][3] = 0.f;
+            if (d < dk)
+                ld4<DT>(kcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dk) + d, kreg[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < VT; ++i) {
+            const int e = tid + 256 * i, row = e / (DVP / 4), d = 4 * (e % (DVP / 4));
+            const int kj = min(k0 + row, total - 1);
+            vreg[i][0] = vreg[i][1] = vreg[i][2] = vreg[i][3] = 0.f;
+            if (d < dv)
+                ld4<DT>(vcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dv) + d, vreg[i]);
+        }
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KT; ++i) {
+            const int e = tid + 256 * i, row = e / (DKP / 4), d = 4 * (e % (DKP / 4));
+            float* kd = ks + row * KLD + d;
+            kd[0] = kreg[i][0]; kd[1] = kreg[i][1]; kd[2] = kreg[i][2]; kd[3] = kreg[i][3];
+        }
+#pragma unroll
+        for (int i = 0; i < VT; ++i) {
+            const int e = tid + 256 * i, row = e / (DVP / 4), d = 4 * (e % (DVP / 4));
+            float* vd = vs + row * DVP + d;
+            vd[0] = vreg[i][0]; vd[1] = vreg[i][1]; vd[2] = vreg[i][2]; vd[3] = vreg[i][3];
+        }
+    };
+    cap_f32x16_t o[VT];
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[t][v] = 0.f;
+    float m_i = NEG_INF, l_i = 0.f;
+
+    const int k_hi = min(total, pos0 + q0 + MQ);
+    int k_lo = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
+    if (chunk > 0) k_lo = max(k_lo, ((pos0 + q0) / chunk) * chunk);
+    k_lo = (k_lo / MK) * MK;
+    const int wq_lo = pos0 + q0 + 32 * wave, wq_hi = wq_lo + 31;
+    const int wc_lo = chunk > 0 ? (wq_lo / chunk) * chunk : 0;     // the wave's first row sees farthest back
+    const int c_lo = chunk > 0 ? (qpos / chunk) * chunk : 0;
+    const int k_last = k_lo + ((k_hi - 1 - k_lo) / MK) * MK;
+    fetch(k_lo);
+    for (int k0 = k_lo; k0 < k_hi; k0 += MK) {
+        __syncthreads();
+        stage();
+        __syncthreads();
+        fetch(min(k0 + MK, k_last));              // (unconditional: the last tile is asked for twice)
+        if (!wave_has_rows || k0 > wq_hi || k0 + MK - 1 < wc_lo || (window > 0 && k0 + MK - 1 <= wq_lo - window))
+            continue;
+        cap_f32x16_t sc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+        const float* kr = ks + col * KLD + half;
+#pragma unroll
+        for (int s2 = 0; s2 < DKP / 2; ++s2)
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[2 * s2], qr[s2], sc, 0, 0, 0);
+        float tm = NEG_INF;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int kj = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+            const bool ok = qrow < len && kj <= qpos && kj >= c_lo && (window <= 0 || kj > qpos - window);
+            sc[v] = ok ? soft_cap(sc[v] * scale, cap, inv_cap) - slope * (float)(qpos - kj) : NEG_INF;
+            tm = fmaxf(tm, sc[v]);
+        }
+        tm = fmaxf(tm, __shfl_xor(tm, 32, ILLM_WAVE));
+        const float m_new = fmaxf(m_i, tm);
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m_i - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            sc[v] = (sc[v] == NEG_INF) ? 0.f : expf(sc[v] - m_new);
+            psum += sc[v];
+        }
+        psum += __shfl_xor(psum, 32, ILLM_WAVE);
+        l_i = l_i * alpha + psum;
+        m_i = m_new;
+#pragma unroll
+        for (int t = 0; t < VT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[t][v] *= alpha;
+        const float* vr = vs + 4 * half * DVP + col;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = 8 * (v >> 2) + (v & 3);         // + 4 * half, in vr
+#pragma unroll
+            for (int t = 0; t < VT; ++t)
+                o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[key * DVP + 32 * t], sc[v], o[t], 0, 0, 0);
+        }
+    }
+    if (qrow < len) {
+        const float inv = 1.0f / l_i;
+        const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
+        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * dv;
+#pragma unroll
+        for (int t = 0; t < VT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int d = 32 * t + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (d < dv) {
+                    float y = o[t][v] * inv;
+                    if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, gb + d)));
+                    st_f(out, DT, ob + d, y);
+                }
+            }
+    }
+}
+
+static int g_attn_cap_mfma = 1;
+extern "C" void illm_set_attn_cap_mfma(int on) { g_attn_cap_mfma = on ? 1 : 0; }
+
 extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int32_t* cu,
                                   const int32_t* seq_slot, const int32_t* seq_start,
                                   const void* kcache, const void* vcache, const int32_t* page_table,
@@ -267,6 +451,25 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
         dv <= 0 || dv > 256 || page_size <= 0 || !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_rows == 0) return ILLM_OK;
+    if (g_attn_cap_mfma && dk <= 128 && dv <= 128 && dk % 4 == 0 && dv % 4 == 0 && q_stride % 4 == 0) {
+        const dim3 grid((max_rows + MQ - 1) / MQ, nh, n_seqs);
+        const int kt = (dk + 31) / 32, vt = (dv + 31) / 32;
+#define GO(DT_, KT_, VT_)                                                                          \
+    hipLaunchKernelGGL((attn_cap_rows_mfma_kernel<DT_, KT_, VT_>), grid, dim3(256), 0, (hipStream_t)stream, \
+                       q, q_stride, out, cu, seq_slot, seq_start, kcache, vcache, page_table, table_stride, \
+                       page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, gate, gate_stride, gate_off)
+#define GO_V(DT_, KT_)                                                                             \
+    switch (vt) { case 1: GO(DT_, KT_, 1); break; case 2: GO(DT_, KT_, 2); break;                  \
+                  case 3: GO(DT_, KT_, 3); break; default: GO(DT_, KT_, 4); break; }
+#define GO_K(DT_)                                                                                  \
+    switch (kt) { case 1: GO_V(DT_, 1) break; case 2: GO_V(DT_, 2) break;                          \
+                  case 3: GO_V(DT_, 3) break; default: GO_V(DT_, 4) break; }
+        if (dt == ILLM_BF16) { GO_K(ILLM_BF16) } else { GO_K(ILLM_F32) }
+#undef GO_K
+#undef GO_V
+#undef GO
+        return illm_launch_status();
+    }
     const size_t lds = ((size_t)(CQ + CK) * (dk + 1) + (size_t)CK * (dv + 1) + CQ * (CK + 1)) * sizeof(float);
     if (lds > 48 * 1024 &&
         hipFuncSetAttribute((const void*)attn_cap_rows_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -381,6 +584,140 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
     if (threadIdx.x == 0) { pp[dv] = mm; pp[dv + 1] = lt; }
 }
 
+// Single tokens with key and value widths of up to 128 in steps of 4.  grid (kv heads x groups of up
+// to 4 query heads that share them, sequences, splits); 256 threads.  Eight lanes take a key: a
+// wave reads 8 rows of keys (and of values) an instruction, whole 32-dim pieces a group, for all the
+// block's query heads at once; a score is 3 exchanges among the eight lanes.  Every group of eight
+// keeps its own running max, sum and weighted values (lane s of a group holds dims 4 s + 32 j ..),
+// the next round's rows are asked for before this round's arithmetic, and the groups, then the waves,
+// are combined at the end in a fixed order.  `partial` as above.
+#define DH 4    // query heads a block takes at most
+template <int DT, int KQ, int VQ>
+__global__ void __launch_bounds__(256)
+attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const void* __restrict__ kcache,
+                             const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
+                             int table_stride, int page_size, int ring, const int32_t* __restrict__ seq_slot,
+                             const int32_t* __restrict__ seq_len, float* __restrict__ partial, int nsplit,
+                             int nh, int nkv, int dk, int dv, float scale, float cap, int window,
+                             const float* __restrict__ slopes, int chunk) {
+    __shared__ float wacc[4][DH][32 * VQ];
+    __shared__ float wm[4][DH], wl[4][DH];
+    const int rep = nh / nkv, per_kv = (rep + DH - 1) / DH;
+    const int kvh = blockIdx.x / per_kv, h0 = kvh * rep + (blockIdx.x % per_kv) * DH;
+    const int hb = min(DH, (kvh + 1) * rep - h0);
+    const int b = blockIdx.y, sp = blockIdx.z;
+    const int w = wave_index(), lane = threadIdx.x & 63, grp = lane >> 3, sub = lane & 7;
+    const int len = seq_len[b], slot = seq_slot[b];
+    int lo_all = window > 0 ? max(0, len - window) : 0;
+    if (chunk > 0) lo_all = max(lo_all, ((len - 1) / chunk) * chunk);
+    const int tiles = (len + 63) / 64, t0 = lo_all / 64;
+    const int per = (tiles - t0 + nsplit - 1) / nsplit;
+    const int k_lo = max(lo_all, (t0 + sp * per) * 64), k_hi = min(len, (t0 + (sp + 1) * per) * 64);
+    const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+    float qv[DH][4 * KQ], acc[DH][4 * VQ], m[DH], l[DH], slope[DH];
+#pragma unroll
+    for (int i = 0; i < DH; ++i) {
+        m[i] = NEG_INF; l[i] = 0.f;
+        slope[i] = (slopes && i < hb) ? slopes[h0 + i] : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4 * VQ; ++c) acc[i][c] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KQ; ++j) {
+            const int d = 4 * sub + 32 * j;
+            qv[i][4 * j] = qv[i][4 * j + 1] = qv[i][4 * j + 2] = qv[i][4 * j + 3] = 0.f;
+            if (i < hb && d < dk) ld4<DT>(q, (size_t)b * q_stride + (size_t)(h0 + i) * dk + d, &qv[i][4 * j]);
+        }
+    }
+    float kn[4 * KQ], vn[4 * VQ];
+    auto fetch = [&](int base) __attribute__((always_inline)) {
+        const int kj = min(base + grp, k_hi - 1);
+        const size_t kat = cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dk);
+        const size_t vat = cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dv);
+#pragma unroll
+        for (int j = 0; j < KQ; ++j) {
+            const int d = 4 * sub + 32 * j;
+            kn[4 * j] = kn[4 * j + 1] = kn[4 * j + 2] = kn[4 * j + 3] = 0.f;
+            if (d < dk) ld4<DT>(kcache, kat + d, &kn[4 * j]);
+        }
+#pragma unroll
+        for (int j = 0; j < VQ; ++j) {
+            const int d = 4 * sub + 32 * j;
+            vn[4 * j] = vn[4 * j + 1] = vn[4 * j + 2] = vn[4 * j + 3] = 0.f;
+            if (d < dv) ld4<DT>(vcache, vat + d, &vn[4 * j]);
+        }
+    };
+    if (k_lo + 8 * w < k_hi) fetch(k_lo + 8 * w);
+    for (int base = k_lo + 8 * w; base < k_hi; base += 32) {
+        float kc[4 * KQ], vc[4 * VQ];
+#pragma unroll
+        for (int c = 0; c < 4 * KQ; ++c) kc[c] = kn[c];
+#pragma unroll
+        for (int c = 0; c < 4 * VQ; ++c) vc[c] = vn[c];
+        if (base + 32 < k_hi) fetch(base + 32);
+        const int kj = base + grp;
+        const bool valid = kj < k_hi;
+#pragma unroll
+        for (int i = 0; i < DH; ++i) {
+            if (i >= hb) continue;
+            float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+            for (int c = 0; c < 4 * KQ; c += 2) {
+                a0 = fmaf(qv[i][c], kc[c], a0);
+                a1 = fmaf(qv[i][c + 1], kc[c + 1], a1);
+            }
+            float d = a0 + a1;
+            d += __shfl_xor(d, 1, ILLM_WAVE);
+            d += __shfl_xor(d, 2, ILLM_WAVE);
+            d += __shfl_xor(d, 4, ILLM_WAVE);
+            const float sc = valid ? soft_cap(d * scale, cap, inv_cap) - slope[i] * (float)(len - 1 - kj) : NEG_INF;
+            const float m_new = fmaxf(m[i], sc);
+            const float alpha = m_new == NEG_INF ? 1.f : expf(m[i] - m_new);
+            const float p = valid ? expf(sc - m_new) : 0.f;
+            l[i] = l[i] * alpha + p;
+            m[i] = m_new;
+#pragma unroll
+            for (int c = 0; c < 4 * VQ; ++c) acc[i][c] = fmaf(p, vc[c], acc[i][c] * alpha);
+        }
+    }
+    // the wave's eight groups into one (every lane of a group holds the same m and l)
+#pragma unroll
+    for (int i = 0; i < DH; ++i) {
+        if (i >= hb) continue;
+        float mm = m[i];
+        mm = fmaxf(mm, __shfl_xor(mm, 8, ILLM_WAVE));
+        mm = fmaxf(mm, __shfl_xor(mm, 16, ILLM_WAVE));
+        mm = fmaxf(mm, __shfl_xor(mm, 32, ILLM_WAVE));
+        const float f = m[i] == NEG_INF ? 0.f : expf(m[i] - mm);
+        float lt = f * l[i];
+        lt += __shfl_xor(lt, 8, ILLM_WAVE);
+        lt += __shfl_xor(lt, 16, ILLM_WAVE);
+        lt += __shfl_xor(lt, 32, ILLM_WAVE);
+#pragma unroll
+        for (int c = 0; c < 4 * VQ; ++c) {
+            float a = f * acc[i][c];
+            a += __shfl_xor(a, 8, ILLM_WAVE);
+            a += __shfl_xor(a, 16, ILLM_WAVE);
+            a += __shfl_xor(a, 32, ILLM_WAVE);
+            if (grp == 0) wacc[w][i][4 * sub + 32 * (c >> 2) + (c & 3)] = a;
+        }
+        if (lane == 0) { wm[w][i] = mm; wl[w][i] = lt; }
+    }
+    __syncthreads();
+    for (int i = 0; i < hb; ++i) {
+        float mm = wm[0][i];
+        for (int x = 1; x < 4; ++x) mm = fmaxf(mm, wm[x][i]);
+        float f[4], lt = 0.f;
+        for (int x = 0; x < 4; ++x) {
+            f[x] = wm[x][i] == NEG_INF ? 0.f : expf(wm[x][i] - mm);
+            lt += f[x] * wl[x][i];
+        }
+        float* pp = partial + (((size_t)b * nh + h0 + i) * nsplit + sp) * (dv + 2);
+        for (int d = threadIdx.x; d < dv; d += 256)
+            pp[d] = f[0] * wacc[0][i][d] + f[1] * wacc[1][i][d] + f[2] * wacc[2][i][d] + f[3] * wacc[3][i][d];
+        if (threadIdx.x == 0) { pp[dv] = mm; pp[dv + 1] = lt; }
+    }
+}
+
 // grid (heads, sequences): combine the splits' partial results in split order.
 __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* __restrict__ out,
                                       int dt, int nsplit, int nh, int dv, const void* __restrict__ gate,
@@ -420,7 +757,25 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (dt == ILLM_BF16)
+    if (g_attn_cap_mfma && dk <= 128 && dv <= 128 && dk % 4 == 0 && dv % 4 == 0 && q_stride % 4 == 0) {
+        const int rep = nh / nkv;
+        const dim3 grid(nkv * ((rep + DH - 1) / DH), B, nsplit);
+        const int kq = (dk + 31) / 32, vq = (dv + 31) / 32;
+#define GO(DT_, KQ_, VQ_)                                                                          \
+    hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_>), grid, dim3(256), 0, st, q, q_stride, \
+                       kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
+                       nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk)
+#define GO_V(DT_, KQ_)                                                                             \
+    switch (vq) { case 1: GO(DT_, KQ_, 1); break; case 2: GO(DT_, KQ_, 2); break;                  \
+                  case 3: GO(DT_, KQ_, 3); break; default: GO(DT_, KQ_, 4); break; }
+#define GO_K(DT_)                                                                                  \
+    switch (kq) { case 1: GO_V(DT_, 1) break; case 2: GO_V(DT_, 2) break;                          \
+                  case 3: GO_V(DT_, 3) break; default: GO_V(DT_, 4) break; }
+        if (dt == ILLM_BF16) { GO_K(ILLM_BF16) } else { GO_K(ILLM_F32) }
+#undef GO_K
+#undef GO_V
+#undef GO
+    } else if (dt == ILLM_BF16)
         hipLaunchKernelGGL(attn_cap_decode_kernel<ILLM_BF16>, dim3(nh, B, nsplit), dim3(256), 0, st, q,
                            q_stride, kcache, vcache, page_table, table_stride, page_size, ring, seq_slot,
                            seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk);

@@ -452,17 +452,30 @@ def test_matrix_memory_kernels_against_plain_torch(dtype):
         _near(got, want, 1e-5)
 
 
+@pytest.mark.parametrize("matrix_cores", [1, 0])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_with_bias_chunks_and_gate_against_plain_torch(dtype):
+def test_attention_with_bias_chunks_and_gate_against_plain_torch(dtype, matrix_cores):
     """Norms over whole q and k, value mixing and the store; then rows over the cache and single
-    tokens with slopes, chunks and the gate, positions on both sides of chunk and page borders."""
+    tokens with slopes, chunks and the gate, positions on both sides of chunk and page borders; the
+    rows on the matrix cores' float32 instruction (widths up to 128 in steps of 4) and on the
+    vector units (every width)."""
+    from inferllm_amd.kernels import ops
+    ops._lib().illm_set_attn_cap_mfma(matrix_cores)
+    try:
+        _attention_cases(dtype)
+    finally:
+        ops._lib().illm_set_attn_cap_mfma(1)
+
+
+def _attention_cases(dtype):
     from inferllm_amd.kernels import ops
     g = torch.Generator().manual_seed(6)
     tol = 1e-5 if dtype == torch.float32 else 2e-2
-    for nh, nkv, dk, dv, chunk, window in ((6, 2, 20, 12, 37, 0), (4, 4, 16, 40, 0, 0), (3, 1, 72, 8, 64, 50)):
-        lens, starts, slots, page, pages = [70, 3, 1], [60, 0, 129], [1, 3, 0], 64, 12
+    for nh, nkv, dk, dv, chunk, window in ((6, 2, 20, 12, 37, 0), (4, 4, 16, 40, 0, 0), (3, 1, 72, 8, 64, 50),
+                                           (4, 2, 128, 128, 45, 0), (2, 2, 34, 130, 33, 0), (8, 2, 100, 36, 0, 0)):
+        lens, starts, slots, page, pages = [150, 3, 1], [60, 0, 129], [1, 3, 0], 64, 20
         T = sum(lens)
-        table = torch.randperm(pages, generator=g)[:12].view(4, 3).to(torch.int32)
+        table = torch.randperm(pages, generator=g).view(4, 5).to(torch.int32)
         cu, seq_slot, row_slot = _packed(lens, slots)
         row_pos = torch.tensor([s + i for n, s in zip(lens, starts) for i in range(n)], dtype=torch.int32)
         width = nh * dk + nkv * dk + nkv * dv + nh * dv
