@@ -59,6 +59,14 @@ int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int planes, siz
                       const void* delta2, int delta2_dt, const void* w, int w_dt, void* out,
                       int out_dt, const int32_t* row_idx, int rows, int E, float eps, void* stream);
 
+// The same with a second weight of w's dtype and a second output of out's (both null: none): the
+// rows normed once and written under two norms' weights, for a block whose two parts each read a
+// norm of their own of the same rows.
+int illm_add2_rmsnorm_two(float* x, const void* delta, int delta_dt, int planes, size_t plane_stride,
+                          const void* delta2, int delta2_dt, const void* w, const void* w2, int w_dt,
+                          void* out, void* out2, int out_dt, const int32_t* row_idx, int rows, int E,
+                          float eps, void* stream);
+
 // out[t, f] = silu(gate_up[t, f]) * gate_up[t, F + f].
 int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream);
 

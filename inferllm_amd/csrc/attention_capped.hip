@@ -629,10 +629,17 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
         }
     }
     float kn[4 * KQ], vn[4 * VQ];
-    auto fetch = [&](int base) __attribute__((always_inline)) {
+    // the page of a round's key is looked up a round before its rows are asked for, so that a round
+    // waits for one trip to memory, not for two in a row
+    auto page_of = [&](int base) __attribute__((always_inline)) {
+        int lp = min(base + grp, k_hi - 1) / page_size;
+        if (ring > 0) lp %= ring;
+        return page_table[(size_t)slot * table_stride + lp];
+    };
+    auto fetch = [&](int base, int page) __attribute__((always_inline)) {
         const int kj = min(base + grp, k_hi - 1);
-        const size_t kat = cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dk);
-        const size_t vat = cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dv);
+        const size_t row = ((size_t)page * nkv + kvh) * page_size + (kj % page_size);
+        const size_t kat = row * dk, vat = row * dv;
 #pragma unroll
         for (int j = 0; j < KQ; ++j) {
             const int d = 4 * sub + 32 * j;
@@ -646,14 +653,21 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
             if (d < dv) ld4<DT>(vcache, vat + d, &vn[4 * j]);
         }
     };
-    if (k_lo + 8 * w < k_hi) fetch(k_lo + 8 * w);
+    int page_next = 0;
+    if (k_lo + 8 * w < k_hi) {
+        fetch(k_lo + 8 * w, page_of(k_lo + 8 * w));
+        page_next = page_of(k_lo + 8 * w + 32);
+    }
     for (int base = k_lo + 8 * w; base < k_hi; base += 32) {
         float kc[4 * KQ], vc[4 * VQ];
 #pragma unroll
         for (int c = 0; c < 4 * KQ; ++c) kc[c] = kn[c];
 #pragma unroll
         for (int c = 0; c < 4 * VQ; ++c) vc[c] = vn[c];
-        if (base + 32 < k_hi) fetch(base + 32);
+        if (base + 32 < k_hi) {
+            fetch(base + 32, page_next);
+            page_next = page_of(base + 64);
+        }
         const int kj = base + grp;
         const bool valid = kj < k_hi;
 #pragma unroll

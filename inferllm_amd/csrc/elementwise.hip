@@ -165,9 +165,32 @@ __global__ void gelu_tanh_kernel(const void* __restrict__ x, void* __restrict__ 
     st_f(out, dt, i, 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))));
 }
 
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// bfloat16 with n % 8 == 0: 8 values (16 bytes) a thread
+__global__ void __launch_bounds__(256)
+gelu_tanh_bf16x8_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out, size_t n8) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const uint4 v = ((const uint4*)x)[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        o[k] = pack_bf16x2(gelu_tanh_f(__uint_as_float(w[k] << 16)), gelu_tanh_f(__uint_as_float(w[k] & 0xffff0000u)));
+    ((uint4*)out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 extern "C" int illm_gelu_tanh(const void* x, void* out, int dt, size_t n, void* stream) {
     if (!illm_dtype_ok(dt)) return ILLM_ERR_ARG;
     if (n == 0) return ILLM_OK;
+    if (dt == ILLM_BF16 && n % 8 == 0 && n / 8 / 256 < 0x7fffffffu) {
+        hipLaunchKernelGGL(gelu_tanh_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, (const bf16_t*)x, (bf16_t*)out, n / 8);
+        return illm_launch_status();
+    }
     hipLaunchKernelGGL(gelu_tanh_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, x, out, dt, n);
     return illm_launch_status();
@@ -190,7 +213,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
                                    const void* __restrict__ delta2, int delta2_dt,
                                    const void* __restrict__ w, int w_dt,
                                    void* __restrict__ out, int out_dt,
-                                   const int32_t* __restrict__ row_idx, int E, float eps) {
+                                   const int32_t* __restrict__ row_idx, int E, float eps,
+                                   const void* __restrict__ w2, void* __restrict__ out2) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const int in_row = row_idx ? row_idx[r] : r;
@@ -216,6 +240,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
             v += d;
         }
         st_f(out, out_dt, ob + i, (v * scale) * ld_f(w, w_dt, i));
+        if (out2) st_f(out2, out_dt, ob + i, (v * scale) * ld_f(w2, w_dt, i));
     }
 }
 
@@ -248,7 +273,8 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
                        int planes, size_t plane_stride4, const void* __restrict__ delta2,
                        int delta2_dt,
                        const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
-                       const int32_t* __restrict__ row_idx, int E, float eps) {
+                       const int32_t* __restrict__ row_idx, int E, float eps,
+                       const void* __restrict__ w2, void* __restrict__ out2) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const int in_row = row_idx ? row_idx[r] : r;
@@ -302,17 +328,26 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int i = threadIdx.x + TH * j;
-        if (i < E4)
+        if (i < E4) {
             st4_f(out, out_dt, ob + i,
                   make_float4((v[j].x * scale) * wv[j].x, (v[j].y * scale) * wv[j].y,
                               (v[j].z * scale) * wv[j].z, (v[j].w * scale) * wv[j].w));
+            if (out2) {                               // the same rows under a second norm's weight
+                const float4 w2v = ld4_f(w2, w_dt, i);
+                st4_f(out2, out_dt, ob + i,
+                      make_float4((v[j].x * scale) * w2v.x, (v[j].y * scale) * w2v.y,
+                                  (v[j].z * scale) * w2v.z, (v[j].w * scale) * w2v.w));
+            }
+        }
     }
 }
 
-extern "C" int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
-                                 size_t plane_stride, const void* delta2, int delta2_dt,
-                                 const void* w, int w_dt, void* out, int out_dt,
-                                 const int32_t* row_idx, int rows, int E, float eps, void* stream) {
+extern "C" int illm_add2_rmsnorm_two(float* x, const void* delta, int delta_dt, int planes,
+                                     size_t plane_stride, const void* delta2, int delta2_dt,
+                                     const void* w, const void* w2, int w_dt, void* out, void* out2,
+                                     int out_dt, const int32_t* row_idx, int rows, int E, float eps,
+                                     void* stream) {
+    if ((w2 == nullptr) != (out2 == nullptr)) return ILLM_ERR_ARG;
     if (delta2 && (!delta || !illm_dtype_ok(delta2_dt))) return ILLM_ERR_ARG;
     if (rows < 0 || E <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
         (delta && (!illm_dtype_ok(delta_dt) || planes < 1 ||
@@ -323,7 +358,7 @@ extern "C" int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int 
 #define VEC(NV_, TH_)                                                                         \
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV_, TH_>), dim3(rows), dim3(TH_), 0, st, x,   \
                        delta, delta_dt, planes, plane_stride / 4, delta2, delta2_dt, w, w_dt, out,  \
-                       out_dt, row_idx, E, eps)
+                       out_dt, row_idx, E, eps, w2, out2)
     // few rows (decoding): wide blocks, one group of 4 floats per thread, to shorten the row's
     // critical path; many rows: narrow blocks so that more rows are in flight per CU
     if (E % 4 == 0 && rows <= 128 && E > 1024 && E <= 4096) VEC(1, 1024);
@@ -335,9 +370,17 @@ extern "C" int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int 
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt,
                            planes, plane_stride, delta2, delta2_dt, w, w_dt, out, out_dt, row_idx, E,
-                           eps);
+                           eps, w2, out2);
 #undef VEC
     return illm_launch_status();
+}
+
+extern "C" int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
+                                 size_t plane_stride, const void* delta2, int delta2_dt,
+                                 const void* w, int w_dt, void* out, int out_dt,
+                                 const int32_t* row_idx, int rows, int E, float eps, void* stream) {
+    return illm_add2_rmsnorm_two(x, delta, delta_dt, planes, plane_stride, delta2, delta2_dt, w, nullptr,
+                                 w_dt, out, nullptr, out_dt, row_idx, rows, E, eps, stream);
 }
 
 extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes,

@@ -199,8 +199,11 @@ def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
 
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                out_dtype: torch.dtype, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out_dtype: torch.dtype, row_idx: Optional[torch.Tensor] = None,
+                weight2: Optional[torch.Tensor] = None):
     """RMS norm of the float32 residual rows `x` [T, E] after adding `delta` to them.
+    With `weight2` (of weight's shape and dtype) a pair comes back: the same normed rows under each
+    of the two weights, from one pass over x.
 
     Without `row_idx` the sum is written back to `x`.  With `row_idx` only those
     rows are normed (and `x` is left as it is).  `delta` may be [S, T, E]: the planes of a
@@ -225,12 +228,17 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _need(delta.shape[-2:] == x.shape, "add_rmsnorm: delta must have x's shape")
     rows = T if row_idx is None else row_idx.numel()
     out = torch.empty((rows, E), dtype=out_dtype, device=x.device)
-    _check(_lib().illm_add2_rmsnorm(
+    out2 = None
+    if weight2 is not None:
+        _gpu(weight2)
+        _need(weight2.shape == (E,) and weight2.dtype == weight.dtype, "add_rmsnorm: a second weight like the first")
+        out2 = torch.empty((rows, E), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_add2_rmsnorm_two(
         _p(x), _p(delta), _code(delta) if delta is not None else 0, planes,
         ctypes.c_size_t(T * E), _p(delta2), _code(delta2) if delta2 is not None else 0,
-        _p(weight), _code(weight),
-        _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
-    return out
+        _p(weight), _p(weight2), _code(weight),
+        _p(out), _p(out2), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+    return out if weight2 is None else (out, out2)
 
 
 class StreamWrite:

@@ -71,11 +71,17 @@ class ParallelBlock(Block):
             pending = None                       # its sum is in x already
         if isinstance(pending, tuple) and not getattr(self.mixer_norm, "adds_pairs", False):
             pending = ops.sum_rows(*pending)
-        h = self.mixer_norm.forward(x, pending, ctx)
+        h2 = None
+        if self.feed_forward_norm is not None and hasattr(self.mixer_norm, "forward_with"):
+            both = self.mixer_norm.forward_with(self.feed_forward_norm, x, pending, ctx)   # one pass over x
+            if both is not None:
+                h, h2 = both
+        if h2 is None:
+            h = self.mixer_norm.forward(x, pending, ctx)
+            # a second norm reads the same x, which holds the sum by now
+            h2 = self.feed_forward_norm.forward(x, None, ctx) if self.feed_forward_norm is not None else h
         a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
-        # a second norm reads the same x, which holds the sum by now
-        two = self.feed_forward_norm is not None
-        f = self.feed_forward.forward(self.feed_forward_norm.forward(x, None, ctx) if two else h, ctx)
+        f = self.feed_forward.forward(h2, ctx)
         if f is None:
             return a
         if next_norm is not None and getattr(next_norm, "adds_pairs", False):

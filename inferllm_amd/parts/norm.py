@@ -42,6 +42,14 @@ class RMSNorm(Norm):
     def forward(self, x, delta, ctx: StepContext, row_idx=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, row_idx)
 
+    def forward_with(self, other: "RMSNorm", x, delta, ctx: StepContext):
+        """(this norm's rows, `other`'s rows) of the same x (+ delta) in one pass, or None if the two
+        norms cannot share one (another eps, another precision of the weights)."""
+        if (type(other) is not RMSNorm or other.eps != self.eps or other.size != self.size
+                or other.weight.dtype != self.weight.dtype):
+            return None
+        return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, weight2=other.weight)
+
 
 @register_part("norm", "stream_rms_norm")
 class StreamRMSNorm(Norm):

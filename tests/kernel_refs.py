@@ -24,7 +24,10 @@ def _embed_rows(tokens, table, scale=1.0):
     return table[tokens.long()].to(torch.float32) * scale
 
 
-def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None):
+def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None, weight2=None):
+    if weight2 is not None:
+        first = add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx)
+        return first, add_rmsnorm(x, None, weight2, eps, out_dtype, row_idx)
     if isinstance(delta, (tuple, list)):               # two parts' outputs for the same rows
         delta = delta[0].to(F64) + delta[1].to(F64)
     if delta is not None:

@@ -541,3 +541,18 @@ def test_pair_embedding_and_gelu_against_plain_torch():
     assert torch.equal(l_got.cpu(), l_want)
     x = torch.randn(1000, generator=g) * 3
     _near(ops.gelu_tanh(x.cuda()), R.gelu_tanh(x), 1e-6)
+    xb = (torch.randn(5, 1024, generator=g) * 3).to(torch.bfloat16)           # 8 values a thread
+    _near(ops.gelu_tanh(xb.cuda()), R.gelu_tanh(xb), 1e-2)
+
+
+@pytest.mark.parametrize("E, T", [(90, 3), (2048, 5), (8200, 2)])
+def test_two_norms_of_the_same_rows_in_one_pass(E, T):
+    from inferllm_amd.kernels import ops
+    g = torch.Generator().manual_seed(E)
+    x, a, b = (torch.randn(T, E, generator=g) for _ in range(3))
+    w1, w2 = torch.randn(E, generator=g), torch.randn(E, generator=g)
+    x_want = x.clone()
+    want = R.add_rmsnorm(x_want, (a, b), w1, 1e-5, torch.float32, None, w2)
+    xg = x.cuda()
+    got = ops.add_rmsnorm(xg, (a.cuda(), b.cuda()), w1.cuda(), 1e-5, torch.float32, weight2=w2.cuda())
+    _near(got[0], want[0], 1e-5); _near(got[1], want[1], 1e-5); _near(xg, x_want, 1e-6)
