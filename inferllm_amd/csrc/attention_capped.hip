@@ -270,6 +270,28 @@ typedef float cap_f32x16_t __attribute__((ext_vector_type(16)));
 #define MQ 128  // query rows of a block
 #define MK 32   // keys of a tile
 
+// Four elements as they are stored (8 bytes of bfloat16 or 16 of float32), kept raw while the load
+// is in flight: whoever turns them into floats waits for the load, so that is left to the user.
+typedef uint32_t cap_u32x2_t __attribute__((ext_vector_type(2)));
+template <int DT> struct Raw4;
+template <> struct Raw4<ILLM_BF16> {
+    cap_u32x2_t r;
+    __device__ __forceinline__ void zero() { r.x = r.y = 0u; }
+    __device__ __forceinline__ void load(const void* p, size_t at) { r = *(const cap_u32x2_t*)((const bf16_t*)p + at); }
+    __device__ __forceinline__ void floats(float* x) const {
+        x[0] = __uint_as_float(r.x << 16); x[1] = __uint_as_float(r.x & 0xffff0000u);
+        x[2] = __uint_as_float(r.y << 16); x[3] = __uint_as_float(r.y & 0xffff0000u);
+    }
+};
+template <> struct Raw4<ILLM_F32> {
+    illm_u32x4_t r;
+    __device__ __forceinline__ void zero() { r.x = r.y = r.z = r.w = 0u; }
+    __device__ __forceinline__ void load(const void* p, size_t at) { r = *(const illm_u32x4_t*)((const float*)p + at); }
+    __device__ __forceinline__ void floats(float* x) const {
+        x[0] = __uint_as_float(r.x); x[1] = __uint_as_float(r.y); x[2] = __uint_as_float(r.z); x[3] = __uint_as_float(r.w);
+    }
+};
+
 template <int DT>
 __device__ __forceinline__ void ld4(const void* p, size_t at, float* x) {
     if (DT == ILLM_BF16) {
@@ -322,37 +344,35 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
         }
     }
     // a thread's share of a tile: quads e = tid + 256 i of [32 keys][DKP / 4] and of [32 keys][DVP / 4]
-    float kreg[KT][4], vreg[VT][4];
+    Raw4<DT> kreg[KT], vreg[VT];                   // (raw: turned into floats when they are staged)
     auto fetch = [&](int k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < KT; ++i) {
             const int e = tid + 256 * i, row = e / (DKP / 4), d = 4 * (e % (DKP / 4));
             const int kj = min(k0 + row, total - 1);       // keys past the end: a valid row, masked below
-            kreg[i][0] = kreg[i][1] = kreg[i][2] = kreg[i][3] = 0.f;
+            kreg[i].zero();
             if (d < dk)
-                ld4<DT>(kcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dk) + d, kreg[i]);
+                kreg[i].load(kcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dk) + d);
         }
 #pragma unroll
         for (int i = 0; i < VT; ++i) {
             const int e = tid + 256 * i, row = e / (DVP / 4), d = 4 * (e % (DVP / 4));
             const int kj = min(k0 + row, total - 1);
-            vreg[i][0] = vreg[i][1] = vreg[i][2] = vreg[i][3] = 0.f;
+            vreg[i].zero();
             if (d < dv)
-                ld4<DT>(vcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dv) + d, vreg[i]);
+                vreg[i].load(vcache, cache_row_offset(page_table, table_stride, slot, kj, page_size, ring, nkv, kvh, dv) + d);
         }
     };
     auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < KT; ++i) {
             const int e = tid + 256 * i, row = e / (DKP / 4), d = 4 * (e % (DKP / 4));
-            float* kd = ks + row * KLD + d;
-            kd[0] = kreg[i][0]; kd[1] = kreg[i][1]; kd[2] = kreg[i][2]; kd[3] = kreg[i][3];
+            kreg[i].floats(ks + row * KLD + d);
         }
 #pragma unroll
         for (int i = 0; i < VT; ++i) {
             const int e = tid + 256 * i, row = e / (DVP / 4), d = 4 * (e % (DVP / 4));
-            float* vd = vs + row * DVP + d;
-            vd[0] = vreg[i][0]; vd[1] = vreg[i][1]; vd[2] = vreg[i][2]; vd[3] = vreg[i][3];
+            vreg[i].floats(vs + row * DVP + d);
         }
     };
     cap_f32x16_t o[VT];
@@ -584,14 +604,31 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
     if (threadIdx.x == 0) { pp[dv] = mm; pp[dv + 1] = lt; }
 }
 
-// Single tokens with key and value widths of up to 128 in steps of 4.  grid (kv heads x groups of up
-// to 4 query heads that share them, sequences, splits); 256 threads.  Eight lanes take a key: a
-// wave reads 8 rows of keys (and of values) an instruction, whole 32-dim pieces a group, for all the
-// block's query heads at once; a score is 3 exchanges among the eight lanes.  Every group of eight
-// keeps its own running max, sum and weighted values (lane s of a group holds dims 4 s + 32 j ..),
-// the next round's rows are asked for before this round's arithmetic, and the groups, then the waves,
-// are combined at the end in a fixed order.  `partial` as above.
+// Single tokens with key and value widths of up to 128 in steps of 4 (float32) or 8 (bfloat16).
+// grid (kv heads x groups of up to 4 query heads that share them, sequences, splits); 256 threads.
+// Eight lanes take a key, each 16 bytes of a row at a time (a unit: 4 floats or 8 bfloat16), so a
+// wave reads 8 rows of keys (and of values) an instruction, a whole 128-byte line a row, for all
+// the block's query heads at once; a score is 3 exchanges among the eight lanes.  Every group of
+// eight keeps its own running max, sum and weighted values (lane s of a group holds dims U s + 8 U j
+// ..), the next round's rows are asked for before this round's arithmetic, and the groups, then the
+// waves, are combined at the end in a fixed order.  `partial` as above.
 #define DH 4    // query heads a block takes at most
+template <int DT>
+__device__ __forceinline__ void ld_unit(const void* p, size_t at, float* x) {
+    if (DT == ILLM_BF16) {
+        const uint4 r = *(const uint4*)((const bf16_t*)p + at);
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            x[2 * k] = __uint_as_float(w[k] << 16);
+            x[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+        }
+    } else {
+        const float4 r = *(const float4*)((const float*)p + at);
+        x[0] = r.x; x[1] = r.y; x[2] = r.z; x[3] = r.w;
+    }
+}
+
 template <int DT, int KQ, int VQ>
 __global__ void __launch_bounds__(256)
 attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const void* __restrict__ kcache,
@@ -600,7 +637,9 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
                              const int32_t* __restrict__ seq_len, float* __restrict__ partial, int nsplit,
                              int nh, int nkv, int dk, int dv, float scale, float cap, int window,
                              const float* __restrict__ slopes, int chunk) {
-    __shared__ float wacc[4][DH][32 * VQ];
+    constexpr int U = DT == ILLM_BF16 ? 8 : 4;          // elements of a unit
+    constexpr int NK = U * KQ, NV = U * VQ;             // dims of a key, of a value, a lane holds
+    __shared__ float wacc[4][DH][8 * NV];
     __shared__ float wm[4][DH], wl[4][DH];
     const int rep = nh / nkv, per_kv = (rep + DH - 1) / DH;
     const int kvh = blockIdx.x / per_kv, h0 = kvh * rep + (blockIdx.x % per_kv) * DH;
@@ -614,21 +653,35 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
     const int per = (tiles - t0 + nsplit - 1) / nsplit;
     const int k_lo = max(lo_all, (t0 + sp * per) * 64), k_hi = min(len, (t0 + (sp + 1) * per) * 64);
     const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
-    float qv[DH][4 * KQ], acc[DH][4 * VQ], m[DH], l[DH], slope[DH];
+    float qv[DH][NK], acc[DH][NV], m[DH], l[DH], slope[DH];
 #pragma unroll
     for (int i = 0; i < DH; ++i) {
         m[i] = NEG_INF; l[i] = 0.f;
         slope[i] = (slopes && i < hb) ? slopes[h0 + i] : 0.f;
 #pragma unroll
-        for (int c = 0; c < 4 * VQ; ++c) acc[i][c] = 0.f;
+        for (int c = 0; c < NV; ++c) acc[i][c] = 0.f;
 #pragma unroll
         for (int j = 0; j < KQ; ++j) {
-            const int d = 4 * sub + 32 * j;
-            qv[i][4 * j] = qv[i][4 * j + 1] = qv[i][4 * j + 2] = qv[i][4 * j + 3] = 0.f;
-            if (i < hb && d < dk) ld4<DT>(q, (size_t)b * q_stride + (size_t)(h0 + i) * dk + d, &qv[i][4 * j]);
+            const int d = U * sub + 8 * U * j;
+#pragma unroll
+            for (int c = 0; c < U; ++c) qv[i][U * j + c] = 0.f;
+            if (i < hb && d < dk) ld_unit<DT>(q, (size_t)b * q_stride + (size_t)(h0 + i) * dk + d, &qv[i][U * j]);
         }
     }
-    float kn[4 * KQ], vn[4 * VQ];
+    illm_u32x4_t kn[KQ], vn[VQ];                   // (raw: turned into floats when the round begins)
+    auto unit_floats = [&](const illm_u32x4_t r, float* x) __attribute__((always_inline)) {
+        if (DT == ILLM_BF16) {
+            const uint32_t wd[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                x[2 * k] = __uint_as_float(wd[k] << 16);
+                x[2 * k + 1] = __uint_as_float(wd[k] & 0xffff0000u);
+            }
+        } else {
+            x[0] = __uint_as_float(r.x); x[1] = __uint_as_float(r.y);
+            x[2] = __uint_as_float(r.z); x[3] = __uint_as_float(r.w);
+        }
+    };
     // the page of a round's key is looked up a round before its rows are asked for, so that a round
     // waits for one trip to memory, not for two in a row
     auto page_of = [&](int base) __attribute__((always_inline)) {
@@ -640,17 +693,18 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
         const int kj = min(base + grp, k_hi - 1);
         const size_t row = ((size_t)page * nkv + kvh) * page_size + (kj % page_size);
         const size_t kat = row * dk, vat = row * dv;
+        const size_t esz = DT == ILLM_BF16 ? 2 : 4;
 #pragma unroll
         for (int j = 0; j < KQ; ++j) {
-            const int d = 4 * sub + 32 * j;
-            kn[4 * j] = kn[4 * j + 1] = kn[4 * j + 2] = kn[4 * j + 3] = 0.f;
-            if (d < dk) ld4<DT>(kcache, kat + d, &kn[4 * j]);
+            const int d = U * sub + 8 * U * j;
+            kn[j] = illm_u32x4_t{0u, 0u, 0u, 0u};
+            if (d < dk) kn[j] = *(const illm_u32x4_t*)((const char*)kcache + (kat + d) * esz);
         }
 #pragma unroll
         for (int j = 0; j < VQ; ++j) {
-            const int d = 4 * sub + 32 * j;
-            vn[4 * j] = vn[4 * j + 1] = vn[4 * j + 2] = vn[4 * j + 3] = 0.f;
-            if (d < dv) ld4<DT>(vcache, vat + d, &vn[4 * j]);
+            const int d = U * sub + 8 * U * j;
+            vn[j] = illm_u32x4_t{0u, 0u, 0u, 0u};
+            if (d < dv) vn[j] = *(const illm_u32x4_t*)((const char*)vcache + (vat + d) * esz);
         }
     };
     int page_next = 0;
@@ -659,11 +713,11 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
         page_next = page_of(k_lo + 8 * w + 32);
     }
     for (int base = k_lo + 8 * w; base < k_hi; base += 32) {
-        float kc[4 * KQ], vc[4 * VQ];
+        float kc[NK], vc[NV];
 #pragma unroll
-        for (int c = 0; c < 4 * KQ; ++c) kc[c] = kn[c];
+        for (int j = 0; j < KQ; ++j) unit_floats(kn[j], &kc[U * j]);
 #pragma unroll
-        for (int c = 0; c < 4 * VQ; ++c) vc[c] = vn[c];
+        for (int j = 0; j < VQ; ++j) unit_floats(vn[j], &vc[U * j]);
         if (base + 32 < k_hi) {
             fetch(base + 32, page_next);
             page_next = page_of(base + 64);
@@ -675,7 +729,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
             if (i >= hb) continue;
             float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-            for (int c = 0; c < 4 * KQ; c += 2) {
+            for (int c = 0; c < NK; c += 2) {
                 a0 = fmaf(qv[i][c], kc[c], a0);
                 a1 = fmaf(qv[i][c + 1], kc[c + 1], a1);
             }
@@ -690,7 +744,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
             l[i] = l[i] * alpha + p;
             m[i] = m_new;
 #pragma unroll
-            for (int c = 0; c < 4 * VQ; ++c) acc[i][c] = fmaf(p, vc[c], acc[i][c] * alpha);
+            for (int c = 0; c < NV; ++c) acc[i][c] = fmaf(p, vc[c], acc[i][c] * alpha);
         }
     }
     // the wave's eight groups into one (every lane of a group holds the same m and l)
@@ -707,12 +761,12 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
         lt += __shfl_xor(lt, 16, ILLM_WAVE);
         lt += __shfl_xor(lt, 32, ILLM_WAVE);
 #pragma unroll
-        for (int c = 0; c < 4 * VQ; ++c) {
+        for (int c = 0; c < NV; ++c) {
             float a = f * acc[i][c];
             a += __shfl_xor(a, 8, ILLM_WAVE);
             a += __shfl_xor(a, 16, ILLM_WAVE);
             a += __shfl_xor(a, 32, ILLM_WAVE);
-            if (grp == 0) wacc[w][i][4 * sub + 32 * (c >> 2) + (c & 3)] = a;
+            if (grp == 0) wacc[w][i][U * sub + 8 * U * (c / U) + (c % U)] = a;
         }
         if (lane == 0) { wm[w][i] = mm; wl[w][i] = lt; }
     }
@@ -771,10 +825,11 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (g_attn_cap_mfma && dk <= 128 && dv <= 128 && dk % 4 == 0 && dv % 4 == 0 && q_stride % 4 == 0) {
+    const int unit = dt == ILLM_BF16 ? 8 : 4;
+    if (g_attn_cap_mfma && dk <= 128 && dv <= 128 && dk % unit == 0 && dv % unit == 0 && q_stride % unit == 0) {
         const int rep = nh / nkv;
         const dim3 grid(nkv * ((rep + DH - 1) / DH), B, nsplit);
-        const int kq = (dk + 31) / 32, vq = (dv + 31) / 32;
+        const int kq = (dk + 8 * unit - 1) / (8 * unit), vq = (dv + 8 * unit - 1) / (8 * unit);
 #define GO(DT_, KQ_, VQ_)                                                                          \
     hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_>), grid, dim3(256), 0, st, q, q_stride, \
                        kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
