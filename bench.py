@@ -438,7 +438,7 @@ def sabipel_config(width, heads, kv_heads, layers, chunk=1024, vocab=32000):
     mlp = {"kind": "dense", "ff": 4 * width}
     kinds = [("mamba2", ssm), ("attention", att), ("mlstm", mem), ("attention", att)]
     return {"architecture": "Sabipel", "vocab": vocab, "width": width, "max_positions": 8192,
-            "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 37, "mul_cur": 11}},
             "layers": [{"type": kinds[i % 4][0], "mixer": dict(kinds[i % 4][1]), "mlp": dict(mlp)}
                        for i in range(layers)]}
 

@@ -356,7 +356,7 @@ def test_a_conversation_in_one_slot(tmp_path):
     eng.cache.check()
 
 
-# ------------------------------------------------------------------ kernels alone, against their plain contracts
+# ------------------------------------------------------------------ kernels alone, against their plain torch stand-ins
 def _cuda(*ts):
     return [t.cuda() if t is not None else None for t in ts]
 

@@ -1,5 +1,5 @@
 """Sabipel through the step function, the cache and the model wiring on the CPU, with the GPU
-kernels replaced by their plain torch contracts (tests/kernel_refs.py): packing, page tables, the
+kernels replaced by their plain torch stand-ins (tests/kernel_refs.py): packing, page tables, the
 states' slots (cleared when handed out, carried from step to step), the convolution's tail and the
 token before a step's first over portions of one and two tokens, values handed from layer to layer,
 which rows get logits."""
