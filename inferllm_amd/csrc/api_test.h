@@ -45,6 +45,8 @@ void illm_set_rows_a_launch(int rows);
 // illm_attn_cap_rows: 0 sends every size to the kernel on the vector units, which sizes beyond 128
 // or not in steps of 4 use, instead of the one on the matrix cores' float32 instruction (default 1).
 void illm_set_attn_cap_mfma(int on);
+// illm_attn_cap_decode, eight lanes a key: query heads of a kv head that a block takes, 4 (default) or 2.
+void illm_set_attn_cap_heads(int n);
 
 #ifdef __cplusplus
 }

@@ -458,6 +458,8 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
 
 static int g_attn_cap_mfma = 1;
 extern "C" void illm_set_attn_cap_mfma(int on) { g_attn_cap_mfma = on ? 1 : 0; }
+static int g_attn_cap_heads = 4;
+extern "C" void illm_set_attn_cap_heads(int n) { g_attn_cap_heads = n == 2 ? 2 : 4; }
 
 extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int32_t* cu,
                                   const int32_t* seq_slot, const int32_t* seq_start,
@@ -612,7 +614,11 @@ attn_cap_decode_kernel(const void* __restrict__ q, int q_stride, const void* __r
 // eight keeps its own running max, sum and weighted values (lane s of a group holds dims U s + 8 U j
 // ..), the next round's rows are asked for before this round's arithmetic, and the groups, then the
 // waves, are combined at the end in a fixed order.  `partial` as above.
-#define DH 4    // query heads a block takes at most
+template <int CTRL>
+__device__ __forceinline__ float cap_dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
 template <int DT>
 __device__ __forceinline__ void ld_unit(const void* p, size_t at, float* x) {
     if (DT == ILLM_BF16) {
@@ -629,14 +635,15 @@ __device__ __forceinline__ void ld_unit(const void* p, size_t at, float* x) {
     }
 }
 
-template <int DT, int KQ, int VQ>
+template <int DT, int KQ, int VQ, int DH>        // DH: query heads a block takes at most
 __global__ void __launch_bounds__(256)
 attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const void* __restrict__ kcache,
                              const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                              int table_stride, int page_size, int ring, const int32_t* __restrict__ seq_slot,
                              const int32_t* __restrict__ seq_len, float* __restrict__ partial, int nsplit,
                              int nh, int nkv, int dk, int dv, float scale, float cap, int window,
-                             const float* __restrict__ slopes, int chunk) {
+                             const float* __restrict__ slopes, int chunk, void* __restrict__ out,
+                             const void* __restrict__ gate, int gate_stride, int gate_off) {
     constexpr int U = DT == ILLM_BF16 ? 8 : 4;          // elements of a unit
     constexpr int NK = U * KQ, NV = U * VQ;             // dims of a key, of a value, a lane holds
     __shared__ float wacc[4][DH][8 * NV];
@@ -733,10 +740,12 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
                 a0 = fmaf(qv[i][c], kc[c], a0);
                 a1 = fmaf(qv[i][c + 1], kc[c + 1], a1);
             }
+            // the sum over the group's eight lanes by data-parallel moves (no trip through LDS):
+            // lanes 1 0 3 2 of every four, lanes 2 3 0 1, then the other four of the eight (mirrored)
             float d = a0 + a1;
-            d += __shfl_xor(d, 1, ILLM_WAVE);
-            d += __shfl_xor(d, 2, ILLM_WAVE);
-            d += __shfl_xor(d, 4, ILLM_WAVE);
+            d += cap_dpp<0xB1>(d);
+            d += cap_dpp<0x4E>(d);
+            d += cap_dpp<0x141>(d);
             const float sc = valid ? soft_cap(d * scale, cap, inv_cap) - slope[i] * (float)(len - 1 - kj) : NEG_INF;
             const float m_new = fmaxf(m[i], sc);
             const float alpha = m_new == NEG_INF ? 1.f : expf(m[i] - m_new);
@@ -778,6 +787,16 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
         for (int x = 0; x < 4; ++x) {
             f[x] = wm[x][i] == NEG_INF ? 0.f : expf(wm[x][i] - mm);
             lt += f[x] * wl[x][i];
+        }
+        if (nsplit == 1) {                              // the one range is the whole result: no merge
+            const float inv = 1.0f / lt;
+            for (int d = threadIdx.x; d < dv; d += 256) {
+                float y = (f[0] * wacc[0][i][d] + f[1] * wacc[1][i][d] + f[2] * wacc[2][i][d] + f[3] * wacc[3][i][d]) * inv;
+                if (gate)
+                    y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, (size_t)b * gate_stride + gate_off + (size_t)(h0 + i) * dv + d)));
+                st_f(out, DT, ((size_t)b * nh + h0 + i) * dv + d, y);
+            }
+            continue;
         }
         float* pp = partial + (((size_t)b * nh + h0 + i) * nsplit + sp) * (dv + 2);
         for (int d = threadIdx.x; d < dv; d += 256)
@@ -827,16 +846,23 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
     hipStream_t st = (hipStream_t)stream;
     const int unit = dt == ILLM_BF16 ? 8 : 4;
     if (g_attn_cap_mfma && dk <= 128 && dv <= 128 && dk % unit == 0 && dv % unit == 0 && q_stride % unit == 0) {
-        const int rep = nh / nkv;
-        const dim3 grid(nkv * ((rep + DH - 1) / DH), B, nsplit);
+        // four query heads of a kv head a block (their keys and values are read once), or two where
+        // that is asked for: half the registers, twice the waves a SIMD, the rows read twice
+        const int rep = nh / nkv, dh = g_attn_cap_heads == 2 ? 2 : 4;
+        const dim3 grid(nkv * ((rep + dh - 1) / dh), B, nsplit);
         const int kq = (dk + 8 * unit - 1) / (8 * unit), vq = (dv + 8 * unit - 1) / (8 * unit);
 #define GO(DT_, KQ_, VQ_)                                                                          \
-    hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_>), grid, dim3(256), 0, st, q, q_stride, \
-                       kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
-                       nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk)
+    if (dh == 2)                                                                                   \
+        hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_, 2>), grid, dim3(256), 0, st, q, q_stride, \
+                           kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
+                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off); \
+    else                                                                                           \
+        hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_, 4>), grid, dim3(256), 0, st, q, q_stride, \
+                           kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
+                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off)
 #define GO_V(DT_, KQ_)                                                                             \
-    switch (vq) { case 1: GO(DT_, KQ_, 1); break; case 2: GO(DT_, KQ_, 2); break;                  \
-                  case 3: GO(DT_, KQ_, 3); break; default: GO(DT_, KQ_, 4); break; }
+    switch (vq) { case 1: { GO(DT_, KQ_, 1); } break; case 2: { GO(DT_, KQ_, 2); } break;          \
+                  case 3: { GO(DT_, KQ_, 3); } break; default: { GO(DT_, KQ_, 4); } break; }
 #define GO_K(DT_)                                                                                  \
     switch (kq) { case 1: GO_V(DT_, 1) break; case 2: GO_V(DT_, 2) break;                          \
                   case 3: GO_V(DT_, 3) break; default: GO_V(DT_, 4) break; }
@@ -844,6 +870,7 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
 #undef GO_K
 #undef GO_V
 #undef GO
+        if (nsplit == 1) return illm_launch_status();    // written whole by the kernel itself
     } else if (dt == ILLM_BF16)
         hipLaunchKernelGGL(attn_cap_decode_kernel<ILLM_BF16>, dim3(nh, B, nsplit), dim3(256), 0, st, q,
                            q_stride, kcache, vcache, page_table, table_stride, page_size, ring, seq_slot,

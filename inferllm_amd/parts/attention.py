@@ -338,9 +338,10 @@ class GatedAttention(Mixer):
             for bound in (window, self.chunk):
                 longest = min(longest, bound) if bound else longest
             tiles = max(1, (longest + 63) // 64)
-            # a block takes up to four query heads of a kv head; enough blocks for four a compute unit
+            # a block takes up to four query heads of a kv head; enough blocks for two a compute unit
+            # (measured: more ranges than that cost more in set-up and merging than they hide)
             blocks = ctx.n_seqs * nkv * -(-(nh // nkv) // 4)
-            nsplit = max(1, min(-(-1024 // max(1, blocks)), 16, tiles))
+            nsplit = max(1, min(-(-512 // max(1, blocks)), 16, tiles))
             o = ops.attn_cap_decode(rows, kc, vc, group.table, group.page_size, group.ring, ctx.seq_slot,
                                     ctx.seq_len, nh, nkv, dk, dv, self.scale, self.softcap, window,
                                     nsplit, self.slopes, self.chunk, gate, self.g_off)
