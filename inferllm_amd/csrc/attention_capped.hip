@@ -9,8 +9,9 @@
 // Keys and values live in the paged cache, K [page][kv head][row][dk], V [page][kv head][row][dv],
 // under one page table; a step first stores its rows (`kv_store2`) and then every row attends over
 // the cache at absolute positions, so whole prompts, portions of prompts and single tokens take
-// the same path.  Float32 arithmetic over float32 or bfloat16 storage; bfloat16 prompts with sizes
-// in steps of 16 take the matrix-core kernel below.
+// the same path.  Float32 arithmetic over float32 or bfloat16 storage: widths of up to 128 in steps
+// of 4 (single tokens: of 16 bytes) take the kernels on the matrix cores' float32 instruction and
+// with eight lanes a key, every other width the plain ones on the vector units.
 #include <math.h>
 
 #include "api.h"
