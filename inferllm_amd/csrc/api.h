@@ -411,13 +411,13 @@ int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int
                        const void* vcache, const int32_t* page_table, int table_stride,
                        int page_size, int ring, int n_seqs, int max_rows, int nh, int nkv, int dk,
                        int dv, float scale, float cap, int window, const float* slopes, int chunk,
-                       const void* gate, int gate_stride, int gate_off, void* stream);
+                       const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream);
 int illm_attn_cap_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
                          const void* vcache, const int32_t* page_table, int table_stride,
                          int page_size, int ring, const int32_t* seq_slot, const int32_t* seq_len,
                          float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
                          float scale, float cap, int window, const float* slopes, int chunk,
-                         const void* gate, int gate_stride, int gate_off, void* stream);
+                         const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream);
 // The two calls above also take: `slopes` float32 [nh] (null: none), score -= slopes[h] (i - j);
 // `chunk` > 0, a row sees only the keys j with floor(j / chunk) = floor(i / chunk); `gate` (null: none),
 // rows [., gate_stride] of the queries' dtype, out *= sigmoid(gate[row, gate_off + h dv + d]).
@@ -464,6 +464,74 @@ int illm_memory_prepare(const void* U, int dt, int u_stride, int i_off, int f_of
 int illm_memory_finish(const float* o, const float* em, const void* w, int w_dt, const void* Z,
                        int z_dt, int z_stride, int z_off, void* out, int out_dt, int T, int H, int dv,
                        float eps, void* stream);
+
+// ---- short causal convolutions with a kept tail, a sublayer's own norm, a clamped gate (short_conv.hip)
+// y(t) = (add_input ? in(t) : 0) + bias[c] + sum_j w[c, j] in(t - (taps - 1 - j)), in(t) = X[t, x_off + c]
+// (+ in_bias[c]); inputs before a step's first row from tail [slots, taps - 1, C]; `update_tail` (one
+// row a sequence) moves the tail on in the same launch.  w float32 [C, taps]; bias, in_bias may be null.
+int illm_short_conv(const void* X, int x_dt, int x_stride, int x_off, const float* in_bias,
+                    const float* w, const float* bias, int taps, void* tail, int tail_dt,
+                    const int32_t* row_slot, int add_input, void* out, int out_dt, int out_stride,
+                    int T, int C, int update_tail, void* stream);
+// The last taps - 1 inputs of every sequence of a step into the tail.
+int illm_short_conv_tail(const void* X, int x_dt, int x_stride, int x_off, const float* in_bias,
+                         void* tail, int tail_dt, const int32_t* cu, const int32_t* seq_slot,
+                         int n_seqs, int C, int taps, void* stream);
+// out[r] = gain * a[r] / sqrt(mean(a[r]^2) + eps) * w, float32.
+int illm_rms_rows_gain(const void* a, int a_dt, const void* w, int w_dt, float* out, int rows, int E,
+                       float eps, float gain, void* stream);
+// gate_up [T, 2F]: out = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
+int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, int T, int F, float limit,
+                           float alpha, void* stream);
+
+// ---- attention over a window of tokens and pooled blocks before it (attention_pooled.hip)
+// In place on packed rows [q (nh dk) | .. k at k_off (nkv dk) | v at v_off (nkv dv)]: q and k heads
+// turned by their positions (cos_sin float32 [n_positions, rot / 2, 2]; pairing 0: i with i + rot / 2,
+// 1: 2i with 2i + 1; null: none), then, with `unit_norm`, divided by their root mean square; k and v
+// stored in the paged cache (kcache null: not stored; nkv 0: queries alone).
+int illm_qk_rotate_store(void* rows, int dt, int row_len, int k_off, int v_off, const float* cos_sin,
+                         int rot, int pairing, int n_positions, int unit_norm, float eps,
+                         const int32_t* row_pos, const int32_t* row_slot, void* kcache, void* vcache,
+                         const int32_t* page_table, int table_stride, int page_size, int ring, int T,
+                         int nh, int nkv, int dk, int dv, void* stream);
+// For every row whose position ends a block of `pool` tokens: the block's mean key and value, from
+// the cache, into row (position / pool) of the sequence in kpool, vpool (same layout and page table).
+int illm_pool_store(const int32_t* row_pos, const int32_t* row_slot, const void* kcache,
+                    const void* vcache, void* kpool, void* vpool, int dt, const int32_t* page_table,
+                    int table_stride, int page_size, int T, int nkv, int dk, int dv, int pool,
+                    void* stream);
+// Rows of a step over the cache: position i sees tokens j with 0 <= i - j < window and pooled block b
+// if b pool + pool - 1 <= i - window (pool 0: none).  score = q . k scale head_scale[h] (null: 1).
+int illm_attn_pooled_rows(const void* q, int q_stride, void* out, int dt, const int32_t* cu,
+                          const int32_t* seq_slot, const int32_t* seq_start, const void* kcache,
+                          const void* vcache, const void* kpool, const void* vpool,
+                          const int32_t* page_table, int table_stride, int page_size, int n_seqs,
+                          int max_rows, int nh, int nkv, int dk, int dv, float scale,
+                          const float* head_scale, int window, int pool, void* stream);
+// The same for one new token a sequence, at position seq_len - 1.
+int illm_attn_pooled_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
+                            const void* vcache, const void* kpool, const void* vpool,
+                            const int32_t* page_table, int table_stride, int page_size,
+                            const int32_t* seq_slot, const int32_t* seq_len, int B, int nh, int nkv,
+                            int dk, int dv, float scale, const float* head_scale, int window, int pool,
+                            void* stream);
+
+// ---- gated linear attention and a gated linear recurrent unit (linear_scan.hip)
+// Inputs of the plain gated rule with a decay per key channel: q dk^-1/2, k, v from U; decay =
+// sigmoid(Z + zb)^(1 / tau); weight 1.
+int illm_gla_prepare(const void* U, int dt, int u_stride, int q_off, int k_off, int v_off,
+                     const void* Z, int z_dt, int z_stride, const float* zb, float tau, float* qn,
+                     float* kn, float* vv, float* beta, float* dec, int T, int H, int dk, int dv,
+                     void* stream);
+// a = exp(-rate sigmoid(Wr u + br) softplus(lam)), x = sqrt(1 - a^2) sigmoid(Wi u + bi) u, the maps
+// block-diagonal in nb blocks: Wt float32 [2, nb, C / nb (in), C / nb (out)].
+int illm_lru_gates(const float* u, const float* Wt, const float* br, const float* bi, const float* lam,
+                   float rate, float* a_out, float* x_out, int T, int C, int nb, void* stream);
+// S <- a S + x per channel over every sequence's rows from state [slots, C] and back into it;
+// out = S gelu_tanh(Y[:, y_off + c] + yb[c]).
+int illm_lru_scan(const float* a, const float* x, float* state, const void* Y, int y_dt, int y_stride,
+                  int y_off, const float* yb, void* out, int out_dt, const int32_t* cu,
+                  const int32_t* seq_slot, int n_seqs, int C, void* stream);
 
 #ifdef __cplusplus
 }

@@ -5,7 +5,7 @@
 // a bias by distance, score -= slopes[h] (i - j) (`slopes` null: none); chunks, position i sees only
 // the keys of its own chunk, floor(j / chunk) = floor(i / chunk), counted from the sequence's
 // position 0 (`chunk` <= 0: none); an output gate, out *= sigmoid(gate[row, gate_off + h dv + d])
-// (`gate` null: none).  Positions enter through the bias and the chunks alone.
+// (`gate` null: none; with `gate_heads` one number a head, gate[row, gate_off + h]).  Positions enter through the bias and the chunks alone.
 // Keys and values live in the paged cache, K [page][kv head][row][dk], V [page][kv head][row][dv],
 // under one page table; a step first stores its rows (`kv_store2`) and then every row attends over
 // the cache at absolute positions, so whole prompts, portions of prompts and single tokens take
@@ -153,7 +153,7 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
                      const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                      int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
                      float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
-                     const void* __restrict__ gate, int gate_stride, int gate_off) {
+                     const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads) {
     extern __shared__ float smem[];
     const int kp = dk + 1, vp = dv + 1;
     float* qs = smem;               // [CQ][kp]
@@ -243,13 +243,13 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
     if (qrow < len) {
         const float inv = 1.0f / l_i;
         const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
-        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * dv;
+        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * (gate_heads ? 1 : dv);
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             const int d = g + 8 * k;
             if (d < dv) {
                 float y = acc[k] * inv;
-                if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, gb + d)));
+                if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, gb + (gate_heads ? 0 : d))));
                 st_f(out, dt, ob + d, y);
             }
         }
@@ -313,7 +313,7 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
                           const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                           int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
                           float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
-                          const void* __restrict__ gate, int gate_stride, int gate_off) {
+                          const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads) {
     constexpr int DKP = 32 * KT, DVP = 32 * VT, KLD = DKP + 1;
     __shared__ float ks[MK * KLD];
     __shared__ float vs[MK * DVP];
@@ -442,7 +442,7 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
     if (qrow < len) {
         const float inv = 1.0f / l_i;
         const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
-        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * dv;
+        const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * (gate_heads ? 1 : dv);
 #pragma unroll
         for (int t = 0; t < VT; ++t)
 #pragma unroll
@@ -450,7 +450,7 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
                 const int d = 32 * t + 8 * (v >> 2) + 4 * half + (v & 3);
                 if (d < dv) {
                     float y = o[t][v] * inv;
-                    if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, gb + d)));
+                    if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, gb + (gate_heads ? 0 : d))));
                     st_f(out, DT, ob + d, y);
                 }
             }
@@ -468,8 +468,8 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
                                   int table_stride, int page_size, int ring, int n_seqs, int max_rows,
                                   int nh, int nkv, int dk, int dv, float scale, float cap, int window,
                                   const float* slopes, int chunk, const void* gate, int gate_stride,
-                                  int gate_off, void* stream) {
-    if (gate && (gate_off < 0 || gate_off + nh * dv > gate_stride)) return ILLM_ERR_ARG;
+                                  int gate_off, int gate_heads, void* stream) {
+    if (gate && (gate_off < 0 || gate_off + nh * (gate_heads ? 1 : dv) > gate_stride)) return ILLM_ERR_ARG;
     if (n_seqs < 0 || max_rows < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 ||
         dv <= 0 || dv > 256 || page_size <= 0 || !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
@@ -480,7 +480,7 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
 #define GO(DT_, KT_, VT_)                                                                          \
     hipLaunchKernelGGL((attn_cap_rows_mfma_kernel<DT_, KT_, VT_>), grid, dim3(256), 0, (hipStream_t)stream, \
                        q, q_stride, out, cu, seq_slot, seq_start, kcache, vcache, page_table, table_stride, \
-                       page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, gate, gate_stride, gate_off)
+                       page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, gate, gate_stride, gate_off, gate_heads)
 #define GO_V(DT_, KT_)                                                                             \
     switch (vt) { case 1: GO(DT_, KT_, 1); break; case 2: GO(DT_, KT_, 2); break;                  \
                   case 3: GO(DT_, KT_, 3); break; default: GO(DT_, KT_, 4); break; }
@@ -501,7 +501,7 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
     hipLaunchKernelGGL(attn_cap_rows_kernel, dim3((max_rows + CQ - 1) / CQ, nh, n_seqs), dim3(256), lds,
                        (hipStream_t)stream, q, q_stride, out, dt, cu, seq_slot, seq_start, kcache, vcache,
                        page_table, table_stride, page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes,
-                       chunk, gate, gate_stride, gate_off);
+                       chunk, gate, gate_stride, gate_off, gate_heads);
     return illm_launch_status();
 }
 
@@ -644,7 +644,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
                              const int32_t* __restrict__ seq_len, float* __restrict__ partial, int nsplit,
                              int nh, int nkv, int dk, int dv, float scale, float cap, int window,
                              const float* __restrict__ slopes, int chunk, void* __restrict__ out,
-                             const void* __restrict__ gate, int gate_stride, int gate_off) {
+                             const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads) {
     constexpr int U = DT == ILLM_BF16 ? 8 : 4;          // elements of a unit
     constexpr int NK = U * KQ, NV = U * VQ;             // dims of a key, of a value, a lane holds
     __shared__ float wacc[4][DH][8 * NV];
@@ -794,7 +794,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
             for (int d = threadIdx.x; d < dv; d += 256) {
                 float y = (f[0] * wacc[0][i][d] + f[1] * wacc[1][i][d] + f[2] * wacc[2][i][d] + f[3] * wacc[3][i][d]) * inv;
                 if (gate)
-                    y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, (size_t)b * gate_stride + gate_off + (size_t)(h0 + i) * dv + d)));
+                    y *= 1.0f / (1.0f + expf(-ld_f(gate, DT, (size_t)b * gate_stride + gate_off + (gate_heads ? (size_t)(h0 + i) : (size_t)(h0 + i) * dv + d))));
                 st_f(out, DT, ((size_t)b * nh + h0 + i) * dv + d, y);
             }
             continue;
@@ -809,7 +809,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
 // grid (heads, sequences): combine the splits' partial results in split order.
 __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* __restrict__ out,
                                       int dt, int nsplit, int nh, int dv, const void* __restrict__ gate,
-                                      int gate_stride, int gate_off) {
+                                      int gate_stride, int gate_off, int gate_heads) {
     const int h = blockIdx.x, b = blockIdx.y;
     const float* pp = partial + ((size_t)b * nh + h) * nsplit * (dv + 2);
     float mm = NEG_INF;
@@ -827,7 +827,7 @@ __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* _
             a += (ms == NEG_INF ? 0.f : expf(ms - mm)) * pp[(size_t)s * (dv + 2) + d];
         }
         float y = a * inv;
-        if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, (size_t)b * gate_stride + gate_off + (size_t)h * dv + d)));
+        if (gate) y *= 1.0f / (1.0f + expf(-ld_f(gate, dt, (size_t)b * gate_stride + gate_off + (gate_heads ? (size_t)h : (size_t)h * dv + d))));
         st_f(out, dt, ((size_t)b * nh + h) * dv + d, y);
     }
 }
@@ -838,8 +838,8 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
                                     int ring, const int32_t* seq_slot, const int32_t* seq_len,
                                     float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
                                     float scale, float cap, int window, const float* slopes, int chunk,
-                                    const void* gate, int gate_stride, int gate_off, void* stream) {
-    if (gate && (gate_off < 0 || gate_off + nh * dv > gate_stride)) return ILLM_ERR_ARG;
+                                    const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream) {
+    if (gate && (gate_off < 0 || gate_off + nh * (gate_heads ? 1 : dv) > gate_stride)) return ILLM_ERR_ARG;
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 ||
         page_size <= 0 || nsplit < 1 || nsplit > 65535 || B > 65535 || !illm_dtype_ok(dt) || !partial)
         return ILLM_ERR_ARG;
@@ -856,11 +856,11 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
     if (dh == 2)                                                                                   \
         hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_, 2>), grid, dim3(256), 0, st, q, q_stride, \
                            kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
-                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off); \
+                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off, gate_heads); \
     else                                                                                           \
         hipLaunchKernelGGL((attn_cap_decode_rows8_kernel<DT_, KQ_, VQ_, 4>), grid, dim3(256), 0, st, q, q_stride, \
                            kcache, vcache, page_table, table_stride, page_size, ring, seq_slot, seq_len, partial, \
-                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off)
+                           nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, out, gate, gate_stride, gate_off, gate_heads)
 #define GO_V(DT_, KQ_)                                                                             \
     switch (vq) { case 1: { GO(DT_, KQ_, 1); } break; case 2: { GO(DT_, KQ_, 2); } break;          \
                   case 3: { GO(DT_, KQ_, 3); } break; default: { GO(DT_, KQ_, 4); } break; }
@@ -882,6 +882,6 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
                            seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk);
     if (hipGetLastError() != hipSuccess) return ILLM_ERR_LAUNCH;
     hipLaunchKernelGGL(attn_cap_merge_kernel, dim3(nh, B), dim3(64), 0, st, partial, out, dt, nsplit, nh, dv,
-                       gate, gate_stride, gate_off);
+                       gate, gate_stride, gate_off, gate_heads);
     return illm_launch_status();
 }

@@ -243,3 +243,148 @@ extern "C" int illm_memory_finish(const float* o, const float* em, const void* w
                        z_dt, z_stride, z_off, out, out_dt, H, dv, eps);
     return illm_launch_status();
 }
+
+// ---------------------------------------------------------------- gated linear attention
+// The plain gated rule with a decay per key channel: from the projections U [T, u_stride] (q at
+// q_off, k at k_off, both H dk wide, v at v_off, H dv wide) and the decays' pre-activations
+// Z [T, z_stride] (H dk wide) with their bias zb:
+//   q dk^-1/2, k, v as float32; decay = sigmoid(Z + zb)^(1 / tau) = exp(logsigmoid(Z + zb) / tau);
+//   the token's weight is 1.
+// grid (rows); 256 threads.
+__global__ void __launch_bounds__(256)
+gla_prepare_kernel(const void* __restrict__ U, int dt, int u_stride, int q_off, int k_off, int v_off,
+                   const void* __restrict__ Z, int z_dt, int z_stride, const float* __restrict__ zb,
+                   float inv_tau, float* __restrict__ qn, float* __restrict__ kn,
+                   float* __restrict__ vv, float* __restrict__ beta, float* __restrict__ dec, int H,
+                   int dk, int dv) {
+    const size_t t = blockIdx.x;
+    const float qs = 1.0f / sqrtf((float)dk);
+    for (int e = threadIdx.x; e < H * dk; e += 256) {
+        qn[t * H * dk + e] = ld_f(U, dt, t * u_stride + q_off + e) * qs;
+        kn[t * H * dk + e] = ld_f(U, dt, t * u_stride + k_off + e);
+        dec[t * H * dk + e] = expf(ls_log_sigmoid(ld_f(Z, z_dt, t * z_stride + e) + zb[e]) * inv_tau);
+    }
+    for (int e = threadIdx.x; e < H * dv; e += 256) vv[t * H * dv + e] = ld_f(U, dt, t * u_stride + v_off + e);
+    for (int e = threadIdx.x; e < H; e += 256) beta[t * H + e] = 1.0f;
+}
+
+extern "C" int illm_gla_prepare(const void* U, int dt, int u_stride, int q_off, int k_off, int v_off,
+                                const void* Z, int z_dt, int z_stride, const float* zb, float tau,
+                                float* qn, float* kn, float* vv, float* beta, float* dec, int T, int H,
+                                int dk, int dv, void* stream) {
+    if (T < 0 || H <= 0 || dk <= 0 || dv <= 0 || !illm_dtype_ok(dt) || !illm_dtype_ok(z_dt) || !(tau > 0.f) ||
+        q_off < 0 || k_off < 0 || v_off < 0 || q_off + H * dk > u_stride || k_off + H * dk > u_stride ||
+        v_off + H * dv > u_stride || H * dk > z_stride)
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(gla_prepare_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, U, dt, u_stride,
+                       q_off, k_off, v_off, Z, z_dt, z_stride, zb, 1.0f / tau, qn, kn, vv, beta, dec, H, dk, dv);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- a gated linear recurrent unit
+// Per channel c of `C`, in `nb` equal blocks of cb channels: with u the recurrence's input,
+//   r = sigmoid(Wr[b] u_b + br),  i = sigmoid(Wi[b] u_b + bi)        (square maps within a block)
+//   a = exp(-rate r softplus(lam)),  x = sqrt(1 - a^2) i u
+//   S <- a S + x,   out = S gelu_tanh(Y + yb)
+// lru_gates gives a and x; lru_scan runs the recurrence from the kept state [slots][C] and back
+// into it and multiplies by the other branch.  All float32 but the stored Y and the output.
+//
+// grid (ceil(T / LRU_ROWS), nb); 256 threads over a block's outputs; the rows' inputs go through
+// LDS.  Wt [2][nb][cb in][cb out] float32: the two maps transposed, so that the threads of a wave
+// read neighbouring outputs of one input.
+#define LRU_ROWS 16
+__global__ void __launch_bounds__(256)
+lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, const float* __restrict__ br,
+                 const float* __restrict__ bi, const float* __restrict__ lam, float rate,
+                 float* __restrict__ a_out, float* __restrict__ x_out, int T, int C, int cb) {
+    extern __shared__ float us[];                   // [LRU_ROWS][cb]
+    const int t0 = blockIdx.x * LRU_ROWS, b = blockIdx.y, nb = C / cb;
+    const int rows = min(LRU_ROWS, T - t0);
+    for (int e = threadIdx.x; e < LRU_ROWS * cb; e += 256) {
+        const int r = e / cb, i = e - r * cb;
+        us[e] = r < rows ? u[(size_t)(t0 + r) * C + (size_t)b * cb + i] : 0.f;
+    }
+    __syncthreads();
+    const float* wr = Wt + (size_t)b * cb * cb;
+    const float* wi = Wt + ((size_t)nb + b) * cb * cb;
+    for (int o = threadIdx.x; o < cb; o += 256) {
+        float ar[LRU_ROWS], ai[LRU_ROWS];
+#pragma unroll
+        for (int r = 0; r < LRU_ROWS; ++r) ar[r] = ai[r] = 0.f;
+        for (int i = 0; i < cb; ++i) {
+            const float w1 = wr[(size_t)i * cb + o], w2 = wi[(size_t)i * cb + o];
+#pragma unroll
+            for (int r = 0; r < LRU_ROWS; ++r) {
+                const float x = us[r * cb + i];
+                ar[r] = fmaf(w1, x, ar[r]);
+                ai[r] = fmaf(w2, x, ai[r]);
+            }
+        }
+        const int c = b * cb + o;
+        const float sp = ls_softplus(lam[c]), b1 = br[c], b2 = bi[c];
+#pragma unroll
+        for (int r = 0; r < LRU_ROWS; ++r) {
+            if (r >= rows) continue;
+            const float rg = ls_sigmoid(ar[r] + b1), ig = ls_sigmoid(ai[r] + b2);
+            const float a = expf(-rate * rg * sp);
+            a_out[(size_t)(t0 + r) * C + c] = a;
+            x_out[(size_t)(t0 + r) * C + c] = sqrtf(fmaxf(1.0f - a * a, 0.f)) * ig * us[r * cb + o];
+        }
+    }
+}
+
+extern "C" int illm_lru_gates(const float* u, const float* Wt, const float* br, const float* bi,
+                              const float* lam, float rate, float* a_out, float* x_out, int T, int C,
+                              int nb, void* stream) {
+    if (T < 0 || C <= 0 || nb <= 0 || C % nb || nb > 65535) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    const int cb = C / nb;
+    const size_t lds = (size_t)LRU_ROWS * cb * sizeof(float);
+    if (lds > 64 * 1024) return ILLM_ERR_ARG;
+    if (lds > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)lru_gates_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+        return ILLM_ERR_LAUNCH;
+    hipLaunchKernelGGL(lru_gates_kernel, dim3((T + LRU_ROWS - 1) / LRU_ROWS, nb), dim3(256), lds,
+                       (hipStream_t)stream, u, Wt, br, bi, lam, rate, a_out, x_out, T, C, cb);
+    return illm_launch_status();
+}
+
+__device__ __forceinline__ float ls_gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// grid (sequences, ceil(C / 256)); a thread walks its channel through the sequence's rows.
+__global__ void __launch_bounds__(256)
+lru_scan_kernel(const float* __restrict__ a, const float* __restrict__ x, float* __restrict__ state,
+                const void* __restrict__ Y, int y_dt, int y_stride, int y_off,
+                const float* __restrict__ yb, void* __restrict__ out, int out_dt,
+                const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot, int C) {
+    const int b = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    if (n <= 0) return;
+    const int slot = seq_slot[b];
+    float S = state[(size_t)slot * C + c];
+    const float bias = yb ? yb[c] : 0.f;
+    for (int t = 0; t < n; ++t) {
+        const size_t at = (size_t)(r0 + t) * C + c;
+        S = fmaf(a[at], S, x[at]);
+        const float y = ls_gelu_tanh(ld_f(Y, y_dt, (size_t)(r0 + t) * y_stride + y_off + c) + bias);
+        st_f(out, out_dt, at, S * y);
+    }
+    state[(size_t)slot * C + c] = S;
+}
+
+extern "C" int illm_lru_scan(const float* a, const float* x, float* state, const void* Y, int y_dt,
+                             int y_stride, int y_off, const float* yb, void* out, int out_dt,
+                             const int32_t* cu, const int32_t* seq_slot, int n_seqs, int C, void* stream) {
+    if (n_seqs < 0 || C <= 0 || !illm_dtype_ok(y_dt) || !illm_dtype_ok(out_dt) || y_off < 0 ||
+        y_off + C > y_stride || n_seqs > 65535 * 32)
+        return ILLM_ERR_ARG;
+    if (n_seqs == 0) return ILLM_OK;
+    hipLaunchKernelGGL(lru_scan_kernel, dim3(n_seqs, (C + 255) / 256), dim3(256), 0, (hipStream_t)stream, a,
+                       x, state, Y, y_dt, y_stride, y_off, yb, out, out_dt, cu, seq_slot, C);
+    return illm_launch_status();
+}

@@ -1,0 +1,166 @@
+// A short causal convolution over time on every channel of packed rows, with the inputs before
+// a step's first row kept per sequence:
+//     in(t)  = X[t, x_off + c] (+ in_bias[c])
+//     y(t)   = (add_input ? in(t) : 0) + bias[c] + sum_{j < taps} w[c, j] in(t - (taps - 1 - j))
+// in(t) is zero before a sequence's first token.  A sequence's rows in a step are consecutive; what
+// lies before the step's first row comes from `tail` [slots][taps - 1][C] (the newest input last),
+// which a fresh slot holds as zeros.  A step of single tokens moves the tail on in the same launch
+// (`update_tail`: the thread that has read a channel's taps writes them back); after a step of
+// several tokens a sequence `short_conv_tail` does.  With `in_bias` the inputs are rounded to the
+// tail's storage type wherever they are read, so a row sees the same numbers whether its
+// neighbours came in this step or an earlier one.  Sums are float32 in the order of the taps.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define CONV_MAX_TAPS 8
+
+__device__ __forceinline__ float conv_round(float v, int dt) {
+    return dt == ILLM_BF16 ? bf16_to_f32(f32_to_bf16(v)) : v;
+}
+
+// grid (rows, ceil(C / 256)); 256 threads, one a channel.
+__global__ void __launch_bounds__(256)
+short_conv_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
+                  const float* __restrict__ in_bias, const float* __restrict__ w,
+                  const float* __restrict__ bias, int taps, void* __restrict__ tail, int tail_dt,
+                  const int32_t* __restrict__ row_slot, int add_input, void* __restrict__ out,
+                  int out_dt, int out_stride, int C, int update_tail) {
+    const int r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int K = taps - 1, slot = row_slot[r];
+    int n = 0;                                  // rows of the same sequence right above this one
+    while (n < K && r - n - 1 >= 0 && row_slot[r - n - 1] == slot) ++n;
+    const float ib = in_bias ? in_bias[c] : 0.f;
+    float in[CONV_MAX_TAPS];                    // in[j]: the input taps - 1 - j rows back
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) continue;
+        const int back = K - j;
+        if (back <= n) {
+            const float v = ld_f(X, x_dt, (size_t)(r - back) * x_stride + x_off + c) + ib;
+            in[j] = in_bias ? conv_round(v, tail_dt) : v;
+        } else {
+            in[j] = ld_f(tail, tail_dt, ((size_t)slot * K + (K - (back - n))) * C + c);
+        }
+    }
+    float y = bias ? bias[c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j)
+        if (j < taps) y = fmaf(w[(size_t)c * taps + j], in[j], y);
+    if (add_input) y += in[K];
+    st_f(out, out_dt, (size_t)r * out_stride + c, y);
+    if (update_tail) {
+#pragma unroll
+        for (int j = 1; j < CONV_MAX_TAPS; ++j)
+            if (j < taps) st_f(tail, tail_dt, ((size_t)slot * K + (j - 1)) * C + c, in[j]);
+    }
+}
+
+extern "C" int illm_short_conv(const void* X, int x_dt, int x_stride, int x_off, const float* in_bias,
+                               const float* w, const float* bias, int taps, void* tail, int tail_dt,
+                               const int32_t* row_slot, int add_input, void* out, int out_dt,
+                               int out_stride, int T, int C, int update_tail, void* stream) {
+    if (T < 0 || C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || !illm_dtype_ok(x_dt) ||
+        !illm_dtype_ok(tail_dt) || !illm_dtype_ok(out_dt) || x_off < 0 || x_off + C > x_stride ||
+        out_stride < C || (C + 255) / 256 > 65535)
+        return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(short_conv_kernel, dim3(T, (C + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       X, x_dt, x_stride, x_off, in_bias, w, bias, taps, tail, tail_dt, row_slot,
+                       add_input, out, out_dt, out_stride, C, taps > 1 ? update_tail : 0);
+    return illm_launch_status();
+}
+
+// The last taps - 1 inputs of every sequence of a step into `tail`.  grid (sequences, ceil(C / 256)).
+__global__ void __launch_bounds__(256)
+short_conv_tail_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
+                       const float* __restrict__ in_bias, void* __restrict__ tail, int tail_dt,
+                       const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot, int C, int K) {
+    const int b = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    if (n <= 0) return;
+    const int slot = seq_slot[b];
+    const float ib = in_bias ? in_bias[c] : 0.f;
+    float keep[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= K) continue;
+        const int at = n - K + j;                       // row of the step, or before it
+        keep[j] = at >= 0 ? ld_f(X, x_dt, (size_t)(r0 + at) * x_stride + x_off + c) + ib
+                          : ld_f(tail, tail_dt, ((size_t)slot * K + (j + n)) * C + c);
+    }
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j)
+        if (j < K) st_f(tail, tail_dt, ((size_t)slot * K + j) * C + c, keep[j]);
+}
+
+extern "C" int illm_short_conv_tail(const void* X, int x_dt, int x_stride, int x_off,
+                                    const float* in_bias, void* tail, int tail_dt, const int32_t* cu,
+                                    const int32_t* seq_slot, int n_seqs, int C, int taps, void* stream) {
+    if (n_seqs < 0 || C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || !illm_dtype_ok(x_dt) ||
+        !illm_dtype_ok(tail_dt) || x_off < 0 || x_off + C > x_stride || (C + 255) / 256 > 65535)
+        return ILLM_ERR_ARG;
+    if (n_seqs == 0 || taps == 1) return ILLM_OK;
+    hipLaunchKernelGGL(short_conv_tail_kernel, dim3(n_seqs, (C + 255) / 256), dim3(256), 0,
+                       (hipStream_t)stream, X, x_dt, x_stride, x_off, in_bias, tail, tail_dt, cu,
+                       seq_slot, C, taps - 1);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- norm of a sublayer's output
+// out[r, :] = gain * a[r, :] / sqrt(mean(a[r]^2) + eps) * w, float32: what a sublayer whose output
+// passes a norm of its own leaves to be added to the residual stream.  grid (rows); 256 threads.
+__global__ void __launch_bounds__(256)
+rms_rows_gain_kernel(const void* __restrict__ a, int a_dt, const void* __restrict__ w, int w_dt,
+                     float* __restrict__ out, int E, float eps, float gain) {
+    __shared__ float red[16];
+    const size_t base = (size_t)blockIdx.x * E;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < E; i += 256) {
+        const float v = ld_f(a, a_dt, base + i);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+    for (int i = threadIdx.x; i < E; i += 256)
+        out[base + i] = gain * (ld_f(a, a_dt, base + i) * inv * ld_f(w, w_dt, i));
+}
+
+extern "C" int illm_rms_rows_gain(const void* a, int a_dt, const void* w, int w_dt, float* out,
+                                  int rows, int E, float eps, float gain, void* stream) {
+    if (rows < 0 || E <= 0 || !illm_dtype_ok(a_dt) || !illm_dtype_ok(w_dt)) return ILLM_ERR_ARG;
+    if (rows == 0) return ILLM_OK;
+    hipLaunchKernelGGL(rms_rows_gain_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, a, a_dt, w,
+                       w_dt, out, E, eps, gain);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- clamped gate * (up + 1)
+// gate_up [T, 2F] = [gate | up]: g = min(gate, limit), u = clamp(up, -limit, limit),
+// out = g sigmoid(alpha g) (u + 1).  grid (ceil(F / 256), rows).
+__global__ void __launch_bounds__(256)
+clamped_swish_mul_kernel(const void* __restrict__ gu, void* __restrict__ out, int dt, int F,
+                         float limit, float alpha) {
+    const size_t t = blockIdx.y;
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    if (f >= F) return;
+    const float g = fminf(ld_f(gu, dt, t * 2 * F + f), limit);
+    const float u = fminf(fmaxf(ld_f(gu, dt, t * 2 * F + F + f), -limit), limit);
+    st_f(out, dt, t * F + f, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+}
+
+extern "C" int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, int T, int F,
+                                      float limit, float alpha, void* stream) {
+    if (T < 0 || F <= 0 || !illm_dtype_ok(dt) || !(limit > 0.f)) return ILLM_ERR_ARG;
+    const size_t esz = dt == ILLM_BF16 ? 2 : 4;
+    for (int t0 = 0; t0 < T; t0 += 65535) {
+        const int rows = T - t0 < 65535 ? T - t0 : 65535;
+        hipLaunchKernelGGL(clamped_swish_mul_kernel, dim3((F + 255) / 256, rows), dim3(256), 0,
+                           (hipStream_t)stream, (const void*)((const char*)gate_up + (size_t)t0 * 2 * F * esz),
+                           (void*)((char*)out + (size_t)t0 * F * esz), dt, F, limit, alpha);
+    }
+    return illm_launch_status();
+}

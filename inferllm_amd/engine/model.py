@@ -114,6 +114,12 @@ class DecoderModel:
             spec = self.layers[e.layer].mixer.state_spec()
             if spec is not None:
                 out[e.cache_line] = spec
+        # what a block arrangement keeps itself (the inputs a convolution in front of its sublayers
+        # still needs): one state per run of the schedule, since runs may share a cache line
+        for i, e in enumerate(self.schedule):
+            own = getattr(self.layers[e.layer], "state_spec", lambda: None)()
+            if own is not None:
+                out[("block", i)] = own
         return out
 
     # ------------------------------------------------------------ compute
@@ -126,6 +132,7 @@ class DecoderModel:
         pending = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
+            ctx.run = i
             if getattr(layer, "takes_next_norm", False):
                 # the norm that will meet this block's output, for kernels that prepare it; none if
                 # the block that follows does not say that it takes rows prepared for its norm

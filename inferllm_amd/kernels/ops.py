@@ -1504,8 +1504,10 @@ def _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, wha
           and page_table.dim() == 2, f"{what}: cache shape or dtype")
 
 
-def _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, what):
+def _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, what, gate_heads=False):
     _gpu(slopes, gate)
+    if gate_heads:
+        dv = 1
     _need(slopes is None or (slopes.dtype == torch.float32 and slopes.shape == (nh,)),
           f"{what}: slopes float32 [{nh}]")
     _need(gate is None or (gate.dim() == 2 and gate.dtype == q.dtype and gate.shape[0] == q.shape[0]
@@ -1553,14 +1555,15 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
                   page_table: torch.Tensor, page_size: int, ring: int, n_seqs: int, max_rows: int,
                   nh: int, nkv: int, dk: int, dv: int, scale: float, cap: float,
                   window: int, slopes: Optional[torch.Tensor] = None, chunk: int = 0,
-                  gate: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
+                  gate: Optional[torch.Tensor] = None, gate_off: int = 0,
+                  gate_heads: bool = False) -> torch.Tensor:
     """Causal attention of a step's packed rows over the paged cache (which holds the step's own
     keys and values by now): row r of sequence b stands at position seq_start[b] + r; scores
     cap tanh(q . k scale / cap) (cap 0: none); queries and keys of width dk, values of dv.
     `slopes` float32 [nh]: score -= slopes[h] (i - j).  `chunk` > 0: a row sees only the keys of its
-    own chunk of positions.  `gate` [T, n] (columns gate_off ..): out *= sigmoid(gate).
-    Returns [T, nh dv]."""
-    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_rows")
+    own chunk of positions.  `gate` [T, n] (columns gate_off ..): out *= sigmoid(gate), one
+    number a head and value dim, or with `gate_heads` one a head.  Returns [T, nh dv]."""
+    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_rows", gate_heads)
     _gpu(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
     _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_rows")
@@ -1569,7 +1572,7 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
         _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh, nkv,
         dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk), _p(gate),
-        gate.shape[1] if gate is not None else 0, gate_off, _stream()),
+        gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _stream()),
         f"attn_cap_rows (sizes {dk}, {dv})")
     return out
 
@@ -1578,10 +1581,11 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                     page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
                     seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
                     cap: float, window: int, nsplit: int, slopes: Optional[torch.Tensor] = None,
-                    chunk: int = 0, gate: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
+                    chunk: int = 0, gate: Optional[torch.Tensor] = None, gate_off: int = 0,
+                    gate_heads: bool = False) -> torch.Tensor:
     """The same attention for one new token per sequence: row b of q against the seq_len[b] keys
     (the new one included) of its slot, the keys cut into `nsplit` ranges.  Returns [B, nh dv]."""
-    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_decode")
+    _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_decode", gate_heads)
     _gpu(q, kcache, vcache, page_table, seq_slot, seq_len)
     B = q.shape[0]
     _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
@@ -1592,7 +1596,7 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(page_table),
         page_table.shape[1], page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh,
         nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk),
-        _p(gate), gate.shape[1] if gate is not None else 0, gate_off, _stream()),
+        _p(gate), gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _stream()),
         f"attn_cap_decode (sizes {dk}, {dv})")
     return out
 
@@ -1790,6 +1794,243 @@ def delta_finish(o: torch.Tensor, weight: torch.Tensor, Z: torch.Tensor, z_off: 
     _check(_lib().illm_delta_finish(_p(o), _p(weight), _code(weight), _p(Z), _code(Z), Z.shape[1], z_off,
                                     DELTA_GATES[gate], _p(out), _code(out), T, H, dv,
                                     ctypes.c_float(eps), _stream()), "delta_finish")
+    return out
+
+
+# ------------------------------------------------------------------ short convolutions, a sublayer's own norm
+def short_conv(X: torch.Tensor, x_off: int, C: int, weight: torch.Tensor, tail: torch.Tensor,
+               row_slot: torch.Tensor, out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None,
+               in_bias: Optional[torch.Tensor] = None, add_input: bool = False,
+               update_tail: bool = False) -> torch.Tensor:
+    """A causal convolution over time on `C` channels of packed rows X [T, n] (columns x_off ..):
+    y(t) = (in(t) if add_input) + bias + sum_j weight[:, j] in(t - (taps - 1 - j)), in = X (+ in_bias);
+    the inputs before a step's first row come from `tail` [slots, taps - 1, C] (zeros in a fresh
+    slot).  weight float32 [C, taps].  `update_tail` (every sequence brings exactly one row): the
+    tail is moved on by that row in the same launch; otherwise `short_conv_tail` does that."""
+    _gpu(X, weight, tail, row_slot, bias, in_bias)
+    T = X.shape[0]
+    _i32(row_slot, T)
+    _need(X.dim() == 2 and 0 <= x_off and x_off + C <= X.shape[1], "short_conv: rows [T, n] with the channels inside")
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[0] == C
+          and 1 <= weight.shape[1] <= 8, "short_conv: weight float32 [C, taps] with 1 to 8 taps")
+    taps = weight.shape[1]
+    _need(tail.dim() == 3 and tail.shape[1:] == (max(taps - 1, 1), C), "short_conv: tail [slots, taps - 1, C]")
+    for b in (bias, in_bias):
+        _need(b is None or (b.dtype == torch.float32 and b.shape == (C,)), "short_conv: biases float32 [C]")
+    out = torch.empty((T, C), dtype=out_dtype, device=X.device)
+    _check(_lib().illm_short_conv(_p(X), _code(X), X.shape[1], x_off, _p(in_bias), _p(weight), _p(bias),
+                                  taps, _p(tail), _code(tail), _p(row_slot), 1 if add_input else 0,
+                                  _p(out), _code(out), C, T, C, 1 if update_tail else 0, _stream()),
+           "short_conv")
+    return out
+
+
+def short_conv_tail(X: torch.Tensor, x_off: int, tail: torch.Tensor, cu_seqlens: torch.Tensor,
+                    seq_slot: torch.Tensor, n_seqs: int, taps: int,
+                    in_bias: Optional[torch.Tensor] = None) -> None:
+    """Keep the last taps - 1 inputs (X's columns from x_off on, + in_bias) of every sequence of the
+    step in `tail` [slots, taps - 1, C]."""
+    _gpu(X, tail, cu_seqlens, seq_slot, in_bias)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
+    C = tail.shape[2]
+    _need(X.dim() == 2 and x_off >= 0 and X.shape[1] >= x_off + C and tail.shape[1] == max(taps - 1, 1),
+          "short_conv_tail: shapes")
+    _need(in_bias is None or (in_bias.dtype == torch.float32 and in_bias.shape == (C,)),
+          "short_conv_tail: in_bias float32 [C]")
+    _check(_lib().illm_short_conv_tail(_p(X), _code(X), X.shape[1], x_off, _p(in_bias), _p(tail),
+                                       _code(tail), _p(cu_seqlens), _p(seq_slot), n_seqs, C, taps,
+                                       _stream()), "short_conv_tail")
+
+
+def rms_rows_gain(a: torch.Tensor, weight: torch.Tensor, eps: float, gain: float) -> torch.Tensor:
+    """float32 [T, E]: gain * a / sqrt(mean(a^2) + eps) * weight, the norm of a sublayer's own output
+    before it is added to the residual stream."""
+    _gpu(a, weight)
+    _need(a.dim() == 2 and weight.shape == (a.shape[1],), "rms_rows_gain: rows [T, E], weight [E]")
+    out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    _check(_lib().illm_rms_rows_gain(_p(a), _code(a), _p(weight), _code(weight), _p(out), a.shape[0],
+                                     a.shape[1], ctypes.c_float(eps), ctypes.c_float(gain), _stream()),
+           "rms_rows_gain")
+    return out
+
+
+SWISH_ALPHA = 1.702
+
+
+def clamped_swish_mul(gate_up: torch.Tensor, limit: float) -> torch.Tensor:
+    """[T, 2F] = [gate | up] -> [T, F]: g sigmoid(1.702 g) (u + 1) with g = min(gate, limit) and
+    u = clamp(up, -limit, limit)."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "clamped_swish_mul: rows [T, 2F]")
+    T, F = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, F), dtype=gate_up.dtype, device=gate_up.device)
+    _check(_lib().illm_clamped_swish_mul(_p(gate_up), _p(out), _code(gate_up), T, F, ctypes.c_float(limit),
+                                         ctypes.c_float(SWISH_ALPHA), _stream()), "clamped_swish_mul")
+    return out
+
+
+# ------------------------------------------------------------------ attention over a window and pooled blocks
+def qk_rotate_store(rows: torch.Tensor, k_off: int, v_off: int, cos_sin: Optional[torch.Tensor],
+                    rot: int, pairing: int, unit_norm: bool, eps: float, row_pos: torch.Tensor,
+                    row_slot: torch.Tensor, kcache: Optional[torch.Tensor],
+                    vcache: Optional[torch.Tensor], page_table: Optional[torch.Tensor], page_size: int,
+                    ring: int, nh: int, nkv: int, dk: int, dv: int) -> None:
+    """In place on packed rows [q (nh dk) | .. k at k_off (nkv dk) | v at v_off (nkv dv)], in float32:
+    the first `rot` dims of every q and k head turned by the row's position (cos_sin float32
+    [positions, rot / 2, 2]; pairing 0: i with i + rot / 2, 1: 2i with 2i + 1), then with `unit_norm`
+    every head divided by its root mean square; k and v stored in the paged cache K [pages, nkv,
+    page_size, dk], V [pages, nkv, page_size, dv] (None: not stored; nkv 0: rows of queries alone)."""
+    _gpu(rows, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
+    T = rows.shape[0]
+    _i32(row_pos, T); _i32(row_slot, T); _i32(page_table)
+    _need(rows.dim() == 2, "qk_rotate_store: rows [T, n]")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[1:] == (rot // 2, 2),
+              "qk_rotate_store: cos_sin float32 [positions, rot / 2, 2]")
+    if kcache is not None:
+        _need(kcache.dtype == rows.dtype and vcache.dtype == rows.dtype
+              and kcache.shape[1:] == (nkv, page_size, dk) and vcache.shape[1:] == (nkv, page_size, dv)
+              and page_table is not None and page_table.dim() == 2, "qk_rotate_store: cache shapes")
+    _check(_lib().illm_qk_rotate_store(
+        _p(rows), _code(rows), rows.shape[1], k_off, v_off, _p(cos_sin), rot if cos_sin is not None else 0,
+        pairing, cos_sin.shape[0] if cos_sin is not None else 0, 1 if unit_norm else 0, ctypes.c_float(eps),
+        _p(row_pos), _p(row_slot), _p(kcache), _p(vcache), _p(page_table),
+        page_table.shape[1] if page_table is not None else 0, page_size, ring, T, nh, nkv, dk, dv,
+        _stream()), "qk_rotate_store")
+
+
+def pool_store(row_pos: torch.Tensor, row_slot: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+               kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+               nkv: int, dk: int, dv: int, pool: int) -> None:
+    """For every row of the step whose position p ends a block of `pool` tokens ((p + 1) % pool == 0):
+    the mean of the block's keys and of its values, as the cache holds them, into row p // pool of
+    the row's sequence in kpool, vpool (laid out and paged like the cache)."""
+    _gpu(row_pos, row_slot, kcache, vcache, kpool, vpool, page_table)
+    T = row_pos.numel()
+    _i32(row_pos); _i32(row_slot, T); _i32(page_table)
+    _need(kcache.shape[1:] == (nkv, page_size, dk) and vcache.shape[1:] == (nkv, page_size, dv)
+          and kpool.shape == kcache.shape and vpool.shape == vcache.shape
+          and len({t.dtype for t in (kcache, vcache, kpool, vpool)}) == 1 and page_table.dim() == 2,
+          "pool_store: cache shapes")
+    _check(_lib().illm_pool_store(_p(row_pos), _p(row_slot), _p(kcache), _p(vcache), _p(kpool), _p(vpool),
+                                  _code(kcache), _p(page_table), page_table.shape[1], page_size, T, nkv, dk,
+                                  dv, int(pool), _stream()), "pool_store")
+
+
+def _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, head_scale, pool, what):
+    _gpu(q, kcache, vcache, kpool, vpool, page_table, head_scale)
+    _i32(page_table)
+    _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, what)
+    _need(head_scale is None or (head_scale.dtype == torch.float32 and head_scale.shape == (nh,)),
+          f"{what}: head_scale float32 [{nh}]")
+    if pool:
+        _need(kpool is not None and vpool is not None and kpool.shape == kcache.shape
+              and vpool.shape == vcache.shape and kpool.dtype == q.dtype and vpool.dtype == q.dtype,
+              f"{what}: pooled rows laid out like the cache")
+
+
+def attn_pooled_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+                     seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                     kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
+                     page_table: torch.Tensor, page_size: int, n_seqs: int, max_rows: int, nh: int,
+                     nkv: int, dk: int, dv: int, scale: float, head_scale: Optional[torch.Tensor],
+                     window: int, pool: int) -> torch.Tensor:
+    """Attention of a step's packed rows over the paged cache (which holds the step's own keys and
+    values, and the pooled rows of the blocks it completed, by now): the row at position i sees
+    tokens j with 0 <= i - j < window and pooled block b if b pool + pool - 1 <= i - window, in one
+    softmax; score = q . k scale head_scale[h].  Returns [T, nh dv]."""
+    _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, head_scale, pool,
+               "attn_pooled_rows")
+    _gpu(cu_seqlens, seq_slot, seq_start)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs)
+    out = torch.empty((q.shape[0], nh * dv), dtype=q.dtype, device=q.device)
+    _check(_lib().illm_attn_pooled_rows(
+        _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
+        _p(vcache), _p(kpool), _p(vpool), _p(page_table), page_table.shape[1], page_size, n_seqs, max_rows,
+        nh, nkv, dk, dv, ctypes.c_float(scale), _p(head_scale), int(window), int(pool), _stream()),
+        f"attn_pooled_rows (sizes {dk}, {dv})")
+    return out
+
+
+def attn_pooled_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                       kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
+                       page_table: torch.Tensor, page_size: int, seq_slot: torch.Tensor,
+                       seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
+                       head_scale: Optional[torch.Tensor], window: int, pool: int) -> torch.Tensor:
+    """The same attention for one new token per sequence, at position seq_len[b] - 1.  Returns [B, nh dv]."""
+    _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, head_scale, pool,
+               "attn_pooled_decode")
+    _gpu(seq_slot, seq_len)
+    B = q.shape[0]
+    _i32(seq_slot, B); _i32(seq_len, B)
+    out = torch.empty((B, nh * dv), dtype=q.dtype, device=q.device)
+    _check(_lib().illm_attn_pooled_decode(
+        _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(kpool), _p(vpool), _p(page_table),
+        page_table.shape[1], page_size, _p(seq_slot), _p(seq_len), B, nh, nkv, dk, dv, ctypes.c_float(scale),
+        _p(head_scale), int(window), int(pool), _stream()), f"attn_pooled_decode (sizes {dk}, {dv})")
+    return out
+
+
+# ------------------------------------------------------------------ gated linear attention, a gated linear recurrent unit
+def gla_prepare(U: torch.Tensor, q_off: int, k_off: int, v_off: int, Z: torch.Tensor,
+                z_bias: torch.Tensor, tau: float, H: int, dk: int, dv: int):
+    """Gated linear attention's float32 inputs for the plain gated rule with a decay per key channel,
+    from the projections U [T, n] (q at q_off and k at k_off, H dk wide; v at v_off, H dv wide) and
+    the decays' pre-activations Z [T, H dk] with their bias: q dk^-1/2, k, v, weight 1 and
+    decay = sigmoid(Z + z_bias)^(1 / tau).
+    Returns (q [T, H, dk], k, v [T, H, dv], weight [T, H], decay [T, H, dk])."""
+    _gpu(U, Z, z_bias)
+    T = U.shape[0]
+    _need(U.dim() == 2 and Z.dim() == 2 and Z.shape == (T, H * dk) and max(q_off, k_off) + H * dk <= U.shape[1]
+          and v_off + H * dv <= U.shape[1], "gla_prepare: projections too narrow")
+    _need(z_bias.dtype == torch.float32 and z_bias.shape == (H * dk,), "gla_prepare: z_bias float32 [H dk]")
+    dev = U.device
+    qn = torch.empty((T, H, dk), dtype=torch.float32, device=dev)
+    kn = torch.empty((T, H, dk), dtype=torch.float32, device=dev)
+    vv = torch.empty((T, H, dv), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    dec = torch.empty((T, H, dk), dtype=torch.float32, device=dev)
+    _check(_lib().illm_gla_prepare(_p(U), _code(U), U.shape[1], q_off, k_off, v_off, _p(Z), _code(Z),
+                                   Z.shape[1], _p(z_bias), ctypes.c_float(tau), _p(qn), _p(kn), _p(vv),
+                                   _p(beta), _p(dec), T, H, dk, dv, _stream()), "gla_prepare")
+    return qn, kn, vv, beta, dec
+
+
+def lru_gates(u: torch.Tensor, w_t: torch.Tensor, r_bias: torch.Tensor, i_bias: torch.Tensor,
+              lam: torch.Tensor, rate: float):
+    """The gates of a gated linear recurrent unit from its input u float32 [T, C]: with the two
+    block-diagonal maps `w_t` float32 [2, blocks, C / blocks (in), C / blocks (out)],
+    r = sigmoid(Wr u + r_bias), i = sigmoid(Wi u + i_bias), a = exp(-rate r softplus(lam)) and
+    x = sqrt(1 - a^2) i u.  Returns (a, x), float32 [T, C]."""
+    _gpu(u, w_t, r_bias, i_bias, lam)
+    T, C = u.shape
+    _need(u.dtype == torch.float32 and w_t.dtype == torch.float32 and w_t.dim() == 4 and w_t.shape[0] == 2
+          and w_t.shape[2] == w_t.shape[3] and w_t.shape[1] * w_t.shape[2] == C, "lru_gates: shapes")
+    _need(all(t.dtype == torch.float32 and t.shape == (C,) for t in (r_bias, i_bias, lam)),
+          "lru_gates: biases and lam float32 [C]")
+    a = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    x = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    _check(_lib().illm_lru_gates(_p(u), _p(w_t), _p(r_bias), _p(i_bias), _p(lam), ctypes.c_float(rate),
+                                 _p(a), _p(x), T, C, w_t.shape[1], _stream()), "lru_gates")
+    return a, x
+
+
+def lru_scan(a: torch.Tensor, x: torch.Tensor, state: torch.Tensor, Y: torch.Tensor, y_off: int,
+             y_bias: Optional[torch.Tensor], cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+             n_seqs: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """S <- a S + x per channel over every sequence's rows in order, from `state` float32 [slots, C]
+    and back into it; returns S gelu_tanh(Y[:, y_off ..] + y_bias) as [T, C]."""
+    _gpu(a, x, state, Y, y_bias, cu_seqlens, seq_slot)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
+    T, C = a.shape
+    _need(a.dtype == torch.float32 and x.dtype == torch.float32 and x.shape == a.shape
+          and state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == C
+          and Y.dim() == 2 and Y.shape[0] == T and y_off + C <= Y.shape[1], "lru_scan: shapes")
+    _need(y_bias is None or (y_bias.dtype == torch.float32 and y_bias.shape == (C,)), "lru_scan: y_bias float32 [C]")
+    out = torch.empty((T, C), dtype=out_dtype, device=a.device)
+    _check(_lib().illm_lru_scan(_p(a), _p(x), _p(state), _p(Y), _code(Y), Y.shape[1], y_off, _p(y_bias),
+                                _p(out), _code(out), _p(cu_seqlens), _p(seq_slot), n_seqs, C, _stream()),
+           "lru_scan")
     return out
 
 

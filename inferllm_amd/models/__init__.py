@@ -1,3 +1,3 @@
-from . import kukupel, llama, rabapel, sabipel  # registers Kukupel, LlamaForCausalLM, Rabapel and Sabipel
+from . import dotorax, kukupel, llama, rabapel, sabipel  # registers Dotorax, Kukupel, LlamaForCausalLM, Rabapel and Sabipel
 
-__all__ = ["kukupel", "llama", "rabapel", "sabipel"]
+__all__ = ["dotorax", "kukupel", "llama", "rabapel", "sabipel"]

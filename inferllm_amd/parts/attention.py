@@ -241,7 +241,21 @@ class GatedAttention(Mixer):
     * `value_mix` "source": the layer's values are handed on to later layers of the step;
       "mixed": v <- (1 - lam) v + lam v_source with the stored scalar `value_mix` and the source
       layer's values of the same token (the mixed v is what the cache keeps);
-    * `gate`: the heads' outputs side by side times sigmoid(W_g h) before the output projection.
+    * `gate`: the heads' outputs side by side times sigmoid(W_g h) before the output projection,
+      one number a head and value dim; `gate` "head": one number a head (W_g is [heads, width]);
+    * a position encoding of the layer (the block's `rotary` part): the first `rotary_dim` dims of
+      every q and k head are turned by the position, pairing "half" (i with i + rotary_dim / 2) or
+      "interleaved"; the cache keeps the turned keys;
+    * `qk_norm` "head": after the rotation every q and k head is divided by its own root mean
+      square (`eps`), without a weight;
+    * `head_scale`: the score of head h is multiplied by the stored `head_scale`[h];
+    * `pool` P > 0 (with `window`): beside the last `window` tokens a row sees one pooled key and
+      value for every block of P tokens that lies wholly before its window (block b if
+      b P + P - 1 <= i - window): the means of the block's keys and values as the cache holds them,
+      kept beside the keys and values ("kp", "vp": block b in row b of the sequence's pages);
+      tokens and blocks share one softmax;
+    * `own_kv` False: the layer has no key and value projections and reads the cache line of an
+      earlier layer of the step (the schedule names it with `writes_cache` False).
 
     Scores, softmax, norms and the mixing are float32.  A step stores its keys and values in the
     paged cache first and every row attends over the cache at its position, so prompts, portions
@@ -254,9 +268,19 @@ class GatedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, softmax_scale: Optional[float] = None, softcap: float = 0.0,
                  window: Optional[int] = None, chunk: int = 0, slope_power: float = 0.0,
-                 qk_norm: bool = False, eps: float = 1e-6, value_mix: Optional[str] = None,
-                 gate: bool = False, tensors=None):
+                 qk_norm=False, eps: float = 1e-6, value_mix: Optional[str] = None,
+                 gate=False, head_scale: bool = False, pool: int = 0, own_kv: bool = True, tensors=None):
         super().__init__(tensors)
+        if qk_norm not in (False, True, "head") or gate not in (False, True, "head"):
+            raise ValueError(f"gated attention: qk_norm {qk_norm!r} or gate {gate!r}: False, True or 'head'")
+        if int(pool or 0) and not window:
+            raise ValueError("gated attention: pooled blocks lie before a window; `pool` needs `window`")
+        if (int(pool or 0) or head_scale) and (gate or chunk or softcap or slope_power or value_mix
+                                               or qk_norm is True):
+            raise ValueError("gated attention: pooled blocks and a scale a head go with a window, a rotation "
+                             "and the norm a head, not with a gate, chunks, a cap, slopes or mixed values")
+        if not own_kv and (value_mix or qk_norm is True):
+            raise ValueError("gated attention: a layer that reads another layer's keys mixes and norms none")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if key_dim > 256 or value_dim > 256:
@@ -269,39 +293,51 @@ class GatedAttention(Mixer):
         self.chunk = int(chunk or 0)
         self.scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(self.dk)
         self.softcap, self.slope_power = float(softcap or 0.0), float(slope_power or 0.0)
-        self.qk_norm, self.eps, self.value_mix, self.gate = bool(qk_norm), float(eps), value_mix, bool(gate)
+        self.qk_norm, self.eps, self.value_mix, self.gate = qk_norm, float(eps), value_mix, gate
+        self.has_head_scale, self.pool, self.own_kv = bool(head_scale), int(pool or 0), bool(own_kv)
+        self.gate_width = self.nh * (1 if gate == "head" else self.dv)
         self.k_off = self.nh * self.dk
-        self.v_off = self.k_off + self.nkv * self.dk
-        self.g_off = self.v_off + self.nkv * self.dv
-        self.slopes = self.lam = self.q_norm = self.k_norm = None
+        self.v_off = self.k_off + (self.nkv * self.dk if self.own_kv else 0)
+        self.g_off = self.v_off + (self.nkv * self.dv if self.own_kv else 0)
+        self.slopes = self.lam = self.q_norm = self.k_norm = self.head_scale = None
 
     def shapes(self) -> Dict[str, TensorWant]:
         keep = dict(keep_stored=True)
-        out = {"q": TensorWant((self.nh * self.dk, self.E)), "k": TensorWant((self.nkv * self.dk, self.E)),
-               "v": TensorWant((self.nkv * self.dv, self.E)), "o": TensorWant((self.E, self.nh * self.dv))}
-        if self.qk_norm:
+        out = {"q": TensorWant((self.nh * self.dk, self.E)), "o": TensorWant((self.E, self.nh * self.dv))}
+        if self.own_kv:
+            out.update(k=TensorWant((self.nkv * self.dk, self.E)), v=TensorWant((self.nkv * self.dv, self.E)))
+        if self.has_head_scale:
+            out["head_scale"] = TensorWant((self.nh,), init="ones_normal", **keep)
+        if self.qk_norm is True:
             out["q_norm"] = TensorWant((self.nh * self.dk,), init="ones_normal", **keep)
             out["k_norm"] = TensorWant((self.nkv * self.dk,), init="ones_normal", **keep)
         if self.value_mix == "mixed":
             out["value_mix"] = TensorWant((), **keep)
         if self.gate:
-            out["g"] = TensorWant((self.nh * self.dv, self.E))
+            out["g"] = TensorWant((self.gate_width, self.E))
         return out
 
     def kv_spec(self) -> KVSpec:
         from ..cache.manager import TokenTensor
-        return KVSpec("window" if self.window else "full",
-                      (TokenTensor("k", (self.nkv, self.dk)), TokenTensor("v", (self.nkv, self.dv))),
+        k, v = (self.nkv, self.dk), (self.nkv, self.dv)
+        if self.pool:
+            # every token stays (a block's pooled row is formed from its tokens when the last one
+            # comes), and block b lies in row b of the sequence's own pages
+            return KVSpec("full", (TokenTensor("k", k), TokenTensor("v", v), TokenTensor("kp", k),
+                                   TokenTensor("vp", v)))
+        return KVSpec("window" if self.window else "full", (TokenTensor("k", k), TokenTensor("v", v)),
                       self.window)
 
     def load(self, tensors) -> None:
         take = lambda n: self._take(tensors, n)
-        rows = [take(n) for n in ("q", "k", "v")] + ([take("g")] if self.gate else [])
+        rows = [take(n) for n in (("q", "k", "v") if self.own_kv else ("q",))] + ([take("g")] if self.gate else [])
         self.w_in = ops.decode_weight(_fuse(rows), "plain", self.decode_copies)     # [q | k | v | g]
         self.w_o = ops.decode_weight(take("o").contiguous(), "plain", self.decode_copies)
         dev = take("q").device
-        if self.qk_norm:
+        if self.qk_norm is True:
             self.q_norm, self.k_norm = take("q_norm").contiguous(), take("k_norm").contiguous()
+        if self.has_head_scale:
+            self.head_scale = take("head_scale").to(torch.float32).contiguous()
         if self.value_mix == "mixed":
             self.lam = take("value_mix").to(torch.float32).reshape(1).contiguous()
         if self.slope_power > 0:
@@ -315,24 +351,57 @@ class GatedAttention(Mixer):
         nh, nkv, dk, dv = self.nh, self.nkv, self.dk, self.dv
         kc, vc, group = ctx.cache.kv_line(line)
         window = self.window or 0
+        if writes_cache != self.own_kv:
+            raise ValueError("gated attention: a layer with key and value projections stores them, and "
+                             "one without reads a line that an earlier layer of the step stored")
         rows = ops.linear(h, self.w_in)
-        first, first_off = None, 0
-        if self.value_mix == "mixed":
-            first, first_off, width = ctx.exchange["value_mix_source"]
-            if width != nkv * dv:
-                raise ValueError(f"value mixing: the source layer's values are {width} wide, this layer's {nkv * dv}")
         store = writes_cache
-        ops.qkv_norm_mix_store(rows, self.k_off, self.v_off, self.q_norm, self.k_norm, self.eps,
-                               self.lam if first is not None else None, first, first_off, ctx.row_pos,
-                               ctx.row_slot, kc if store else None, vc if store else None, group.table,
-                               group.page_size, group.ring, nh, nkv, dk, dv)
-        if self.value_mix == "source":
-            ctx.exchange["value_mix_source"] = (rows, self.v_off, nkv * dv)
+        if position is not None or self.qk_norm == "head":
+            # rotation, the norm a head and the store in one pass over the rows
+            table = position.table(ctx.device) if position is not None else None
+            ops.qk_rotate_store(rows, self.k_off, self.v_off, table,
+                                position.rotary_dim if position is not None else 0,
+                                0 if position is None or position.pairing == "half" else 1,
+                                self.qk_norm == "head", self.eps, ctx.row_pos, ctx.row_slot,
+                                kc if store else None, vc if store else None, group.table, group.page_size,
+                                group.ring, nh, nkv if self.own_kv else 0, dk, dv)
+        else:
+            first, first_off = None, 0
+            if self.value_mix == "mixed":
+                first, first_off, width = ctx.exchange["value_mix_source"]
+                if width != nkv * dv:
+                    raise ValueError(f"value mixing: the source layer's values are {width} wide, this layer's {nkv * dv}")
+            ops.qkv_norm_mix_store(rows, self.k_off, self.v_off, self.q_norm, self.k_norm, self.eps,
+                                   self.lam if first is not None else None, first, first_off, ctx.row_pos,
+                                   ctx.row_slot, kc if store else None, vc if store else None, group.table,
+                                   group.page_size, group.ring, nh, nkv, dk, dv)
+            if self.value_mix == "source":
+                ctx.exchange["value_mix_source"] = (rows, self.v_off, nkv * dv)
+        if self.pool or self.has_head_scale:
+            kp = vp = None
+            if self.pool:
+                line_tensors, _ = ctx.cache.token_line(line)
+                kp, vp = line_tensors["kp"], line_tensors["vp"]
+                if store:
+                    ops.pool_store(ctx.row_pos, ctx.row_slot, kc, vc, kp, vp, group.table, group.page_size,
+                                   nkv, dk, dv, self.pool)
+            seen = window or (1 << 30)
+            if ctx.prefill:
+                o = ops.attn_pooled_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, kp, vp,
+                                         group.table, group.page_size, ctx.n_seqs, ctx.max_rows, nh, nkv, dk,
+                                         dv, self.scale, self.head_scale, seen, self.pool)
+            else:
+                o = ops.attn_pooled_decode(rows, kc, vc, kp, vp, group.table, group.page_size, ctx.seq_slot,
+                                           ctx.seq_len, nh, nkv, dk, dv, self.scale, self.head_scale, seen,
+                                           self.pool)
+            return ops.linear(o, self.w_o)
         gate = rows if self.gate else None
+        by_head = self.gate == "head"
         if ctx.prefill:
             o = ops.attn_cap_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, group.table,
                                   group.page_size, group.ring, ctx.n_seqs, ctx.max_rows, nh, nkv, dk, dv,
-                                  self.scale, self.softcap, window, self.slopes, self.chunk, gate, self.g_off)
+                                  self.scale, self.softcap, window, self.slopes, self.chunk, gate, self.g_off,
+                                  by_head)
         else:
             longest = ctx.max_len
             for bound in (window, self.chunk):
@@ -344,5 +413,5 @@ class GatedAttention(Mixer):
             nsplit = max(1, min(-(-512 // max(1, blocks)), 16, tiles))
             o = ops.attn_cap_decode(rows, kc, vc, group.table, group.page_size, group.ring, ctx.seq_slot,
                                     ctx.seq_len, nh, nkv, dk, dv, self.scale, self.softcap, window,
-                                    nsplit, self.slopes, self.chunk, gate, self.g_off)
+                                    nsplit, self.slopes, self.chunk, gate, self.g_off, by_head)
         return ops.linear(o, self.w_o)

@@ -54,6 +54,7 @@ class StepContext:
     # of the longest): work that is cut evenly by sequence is then uneven by block
     ragged: bool = False
     exchange: Dict[Any, Any] = field(default_factory=dict)   # between runs of layers in one step
+    run: int = 0                      # which entry of the model's schedule is running (set by the model)
 
 
 class Part:
@@ -210,6 +211,13 @@ class Block(Part):
 
     def load_own(self, tensors) -> None:
         """Take the arrangement's own tensors (those of `shapes()`); most have none."""
+
+    def state_spec(self):
+        """Fixed-size state per sequence that the arrangement itself keeps (beside its mixer's): a
+        `StateSpec`, a dict name -> StateSpec, or None.  The cache manager holds it under the line
+        ("block", run) for every run of the layer in the schedule; `forward` finds it with
+        `ctx.cache.state_line(("block", ctx.run))`."""
+        return None
 
     def load(self, tensors) -> None:
         self.mixer.position = self.position      # a mixer may lay its matrices out for the encoding

@@ -3,6 +3,7 @@ from __future__ import annotations
 
 import torch
 
+from ..cache.manager import StateSpec
 from ..kernels import ops
 from ..weights.loader import TensorWant
 from .base import Block, StepContext, register_part
@@ -87,6 +88,82 @@ class ParallelBlock(Block):
         if next_norm is not None and getattr(next_norm, "adds_pairs", False):
             return (a, f)
         return ops.sum_rows(a, f)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Block):
+    """Sublayers with a norm in front and a norm of their own behind, a gain on what they add, and
+    a short convolution over time in front of what they read:
+
+        x <- x + gain * post1(mixer(c1(norm1(x))));   x <- x + gain * post2(feed_forward(c2(norm2(x))))
+        c(h)_t = h_t + sum_j w[:, j] h_(t - taps + 1 + j)       (zeros before the sequence; taps 0: c(h) = h)
+
+    The post norms are RMS norms over the width with gain `weight_offset` + stored weight, like the
+    norms in front (which are parts of their own).  The last taps - 1 normed rows of either sublayer
+    are part of a sequence's state, which the arrangement keeps itself ("tail1", "tail2").  What a
+    sublayer adds is formed in float32 and handed to the next norm, which adds it to the stream.
+    A layer whose feed-forward is "none" has the first sublayer alone.
+    """
+
+    graph_safe_prompts = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, position, size: int,
+                 eps: float, gain: float = 1.0, taps: int = 0, weight_offset: float = 0.0, tensors=None):
+        super().__init__(mixer, feed_forward, mixer_norm, feed_forward_norm, position, tensors)
+        self.size, self.eps, self.gain = int(size), float(eps), float(gain)
+        self.taps, self.weight_offset = int(taps), float(weight_offset)
+        if not 0 <= self.taps <= 8:
+            raise ValueError(f"sandwich block: {taps} taps; the kernels take up to 8")
+        self.has_ff = feed_forward_norm is not None
+        self.post = [None, None]
+        self.conv = [None, None]
+
+    def _sublayers(self):
+        return (1, 2) if self.has_ff else (1,)
+
+    def shapes(self):
+        out = {}
+        for q in self._sublayers():
+            out[f"post{q}"] = TensorWant((self.size,), init="normal" if self.weight_offset else "ones_normal",
+                                         keep_stored=True)
+            if self.taps:
+                out[f"conv{q}"] = TensorWant((self.size, self.taps), keep_stored=True)
+        return out
+
+    def state_spec(self):
+        if self.taps < 2:
+            return None
+        return {f"tail{q}": StateSpec((self.taps - 1, self.size), None) for q in self._sublayers()}
+
+    def load_own(self, tensors) -> None:
+        for q in self._sublayers():
+            w = self._take(tensors, f"post{q}")
+            self.post[q - 1] = ((w.to(torch.float32) + self.weight_offset) if self.weight_offset else w).contiguous()
+            if self.taps:
+                self.conv[q - 1] = self._take(tensors, f"conv{q}").to(torch.float32).contiguous()
+
+    def _read(self, h, q: int, ctx: StepContext):
+        """What sublayer q reads: the normed rows plus their convolution over time."""
+        if not self.taps:
+            return h
+        if self.taps == 1:
+            tail = h.new_zeros((1, 1, self.size))
+        else:
+            tail = ctx.cache.state_line(("block", ctx.run))[f"tail{q}"]
+        out = ops.short_conv(h, 0, self.size, self.conv[q - 1], tail, ctx.row_slot, h.dtype,
+                             add_input=True, update_tail=not ctx.prefill)
+        if ctx.prefill and self.taps > 1:
+            ops.short_conv_tail(h, 0, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps)
+        return out
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache):
+        h = self._read(self.mixer_norm.forward(x, pending, ctx), 1, ctx)
+        a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
+        d = ops.rms_rows_gain(a, self.post[0], self.eps, self.gain)
+        if not self.has_ff:
+            return d
+        h2 = self._read(self.feed_forward_norm.forward(x, d, ctx), 2, ctx)
+        return ops.rms_rows_gain(self.feed_forward.forward(h2, ctx), self.post[1], self.eps, self.gain)
 
 
 @register_part("block", "hyper_connections")

@@ -103,6 +103,37 @@ class DenseActivation(FeedForward):
         return ops.linear(act(ops.linear(h, self.w_up)), self.w_down)
 
 
+@register_part("feed_forward", "clamped_gated")
+class ClampedGated(FeedForward):
+    """down(g sigmoid(1.702 g) (u + 1)) with g = min(gate h, limit) and u = clamp(up h, -limit, limit):
+    the clamped activation of the routed experts as a dense feed-forward; gate and up are one
+    fused product."""
+
+    graph_safe_prompts = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, tensors=None):
+        super().__init__(tensors)
+        if not float(limit) > 0:
+            raise ValueError("clamped gated feed-forward: the limit must be positive")
+        self.E, self.F, self.limit = int(hidden_size), int(intermediate_size), float(limit)
+        self.w_gate_up = self.w_down = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        return {"gate": TensorWant((self.F, self.E)), "up": TensorWant((self.F, self.E)),
+                "down": TensorWant((self.E, self.F))}
+
+    def load(self, tensors) -> None:
+        self.w_gate_up = ops.decode_weight(_fuse([self._take(tensors, "gate"), self._take(tensors, "up")]),
+                                           "plain", self.decode_copies)
+        self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous(), "plain", self.decode_copies)
+
+    def tunables(self):
+        return (("plain", self.w_down, {}),)
+
+    def forward(self, h, ctx: StepContext):
+        return ops.linear(ops.clamped_swish_mul(ops.linear(h, self.w_gate_up), self.limit), self.w_down)
+
+
 @register_part("feed_forward", "routed_experts")
 class RoutedExperts(FeedForward):
     """A mixture of gated experts, of which every token uses `top`.

@@ -16,6 +16,8 @@ class RMSNorm(Norm):
 
     src/kern/naive/naive.cpp:186-207 and src/core/op.cpp:37-47; eps is a parameter
     (the reference fixes 1e-6 / 1e-5 at src/graph/llama_like.cpp:78 and src/core/graph.h:163).
+    `weight_offset` c: the stored tensor lies around zero and the gain is c + stored (formed once,
+    in float32, as the tensor is taken).
     """
 
     graph_safe_prompts = True
@@ -25,16 +27,19 @@ class RMSNorm(Norm):
     # added as x + (first + second) in the norm's own kernel
     adds_pairs = True
 
-    def __init__(self, size: int, eps: float, tensors=None):
+    def __init__(self, size: int, eps: float, weight_offset: float = 0.0, tensors=None):
         super().__init__(tensors)
-        self.size, self.eps = int(size), float(eps)
+        self.size, self.eps, self.weight_offset = int(size), float(eps), float(weight_offset)
         self.weight: Optional[torch.Tensor] = None
 
     def shapes(self) -> Dict[str, TensorWant]:
-        return {"weight": TensorWant((self.size,), init="ones_normal", keep_stored=True)}
+        return {"weight": TensorWant((self.size,), init="normal" if self.weight_offset else "ones_normal",
+                                     keep_stored=True)}
 
     def load(self, tensors) -> None:
         self.weight = self._take(tensors, "weight").contiguous()
+        if self.weight_offset:
+            self.weight = (self.weight.to(torch.float32) + self.weight_offset).contiguous()
 
     def rms_params(self):
         return self.weight, self.eps

@@ -462,9 +462,12 @@ def _first_seen(pos, window, chunk):
     return max(first, pos // chunk * chunk) if chunk and chunk > 0 else first
 
 
-def _gated(out_row, gate, r, gate_off):
+def _gated(out_row, gate, r, gate_off, heads=0):
     if gate is None:
         return out_row
+    if heads:                                         # one number a head
+        g = torch.sigmoid(gate[r, gate_off:gate_off + heads].to(F64))
+        return (out_row.view(heads, -1) * g[:, None]).reshape(-1)
     return out_row * torch.sigmoid(gate[r, gate_off:gate_off + out_row.numel()].to(F64))
 
 
@@ -491,7 +494,7 @@ def _cached(kcache, vcache, page_table, slot, first, total, page_size, ring):
 
 def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, page_size, ring,
                   n_seqs, max_rows, nh, nkv, dk, dv, scale, cap, window, slopes=None, chunk=0, gate=None,
-                  gate_off=0):
+                  gate_off=0, gate_heads=False):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(n_seqs):
         s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
@@ -500,19 +503,19 @@ def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table
             first = _first_seen(pos, window, chunk)
             k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, pos + 1, page_size, ring)
             row = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
-            out[s0 + a] = _gated(row, gate, s0 + a, gate_off).to(q.dtype)
+            out[s0 + a] = _gated(row, gate, s0 + a, gate_off, nh if gate_heads else 0).to(q.dtype)
     return out
 
 
 def attn_cap_decode(q, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, dk, dv,
-                    scale, cap, window, nsplit, slopes=None, chunk=0, gate=None, gate_off=0):
+                    scale, cap, window, nsplit, slopes=None, chunk=0, gate=None, gate_off=0, gate_heads=False):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(q.shape[0]):
         n = int(seq_len[b])
         first = _first_seen(n - 1, window, chunk)
         k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, n, page_size, ring)
         row = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
-        out[b] = _gated(row, gate, b, gate_off).to(q.dtype)
+        out[b] = _gated(row, gate, b, gate_off, nh if gate_heads else 0).to(q.dtype)
     return out
 
 
@@ -686,6 +689,175 @@ def gelu_tanh(x):
     return (0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))).to(x.dtype)
 
 
+# ---------------------------------------------------------------- short convolutions, a sublayer's own norm
+def _rows_above(row_slot, r, most):
+    n = 0
+    while n < most and r - n - 1 >= 0 and int(row_slot[r - n - 1]) == int(row_slot[r]):
+        n += 1
+    return n
+
+
+def short_conv(X, x_off, C, weight, tail, row_slot, out_dtype, bias=None, in_bias=None, add_input=False,
+               update_tail=False):
+    T, taps = X.shape[0], weight.shape[1]
+    K = taps - 1
+    x = X[:, x_off:x_off + C].to(F64)
+    if in_bias is not None:
+        x = (x + in_bias.to(F64)).to(tail.dtype).to(F64)      # as the tail would hold them
+    out = torch.zeros(T, C, dtype=F64)
+    for r in range(T):
+        slot, n = int(row_slot[r]), _rows_above(row_slot, r, K)
+        ins = []
+        for j in range(taps):
+            back = K - j
+            ins.append(x[r - back] if back <= n else tail[slot, K - (back - n)].to(F64))
+        y = bias.to(F64).clone() if bias is not None else torch.zeros(C, dtype=F64)
+        for j in range(taps):
+            y = y + weight[:, j].to(F64) * ins[j]
+        out[r] = y + (ins[K] if add_input else 0.0)
+        if update_tail and K:
+            tail[slot] = torch.stack(ins[1:]).to(tail.dtype)
+    return out.to(out_dtype)
+
+
+def short_conv_tail(X, x_off, tail, cu_seqlens, seq_slot, n_seqs, taps, in_bias=None):
+    K, C = taps - 1, tail.shape[2]
+    x = X[:, x_off:x_off + C].to(F64)
+    if in_bias is not None:
+        x = x + in_bias.to(F64)
+    for b in range(n_seqs if K else 0):
+        r0, n, slot = int(cu_seqlens[b]), int(cu_seqlens[b + 1]) - int(cu_seqlens[b]), int(seq_slot[b])
+        if n <= 0:
+            continue
+        old = tail[slot].clone()
+        for j in range(K):
+            at = n - K + j
+            tail[slot, j] = x[r0 + at].to(tail.dtype) if at >= 0 else old[j + n]
+
+
+def rms_rows_gain(a, weight, eps, gain):
+    x = a.to(F64)
+    return (gain * (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(F64))).to(torch.float32)
+
+
+def clamped_swish_mul(gate_up, limit):
+    F = gate_up.shape[1] // 2
+    g = torch.clamp(gate_up[:, :F].to(F64), max=limit)
+    u = torch.clamp(gate_up[:, F:].to(F64), -limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1)).to(gate_up.dtype)
+
+
+# ---------------------------------------------------------------- attention over a window and pooled blocks
+def qk_rotate_store(rows, k_off, v_off, cos_sin, rot, pairing, unit_norm, eps, row_pos, row_slot, kcache,
+                    vcache, page_table, page_size, ring, nh, nkv, dk, dv):
+    half = rot // 2
+    for r in range(rows.shape[0]):
+        for off, heads in ((0, nh), (k_off, nkv)):
+            if not heads:
+                continue
+            x = rows[r, off:off + heads * dk].to(F64).view(heads, dk).clone()
+            if cos_sin is not None and rot:
+                c, s = cos_sin[int(row_pos[r]), :, 0].to(F64), cos_sin[int(row_pos[r]), :, 1].to(F64)
+                ia = torch.arange(half) if pairing == 0 else 2 * torch.arange(half)
+                ib = ia + half if pairing == 0 else ia + 1
+                u, v = x[:, ia].clone(), x[:, ib].clone()
+                x[:, ia], x[:, ib] = u * c - v * s, v * c + u * s
+            if unit_norm:
+                x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+            rows[r, off:off + heads * dk] = x.reshape(-1).to(rows.dtype)
+    if kcache is not None:
+        kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table, page_size, ring, nkv, dk, dv)
+
+
+def pool_store(row_pos, row_slot, kcache, vcache, kpool, vpool, page_table, page_size, nkv, dk, dv, pool):
+    for r in range(row_pos.numel()):
+        pos, slot = int(row_pos[r]), int(row_slot[r])
+        if (pos + 1) % pool:
+            continue
+        b = pos // pool
+        k, v = _cached(kcache, vcache, page_table, slot, b * pool, b * pool + pool, page_size, 0)
+        page, at = cache_offsets(page_table, slot, b, page_size, 0)
+        kpool[page, :, at, :] = k.to(F64).mean(0).to(kpool.dtype)
+        vpool[page, :, at, :] = v.to(F64).mean(0).to(vpool.dtype)
+
+
+def _attend_pooled(q, pos, slot, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, scale,
+                   head_scale, window, pool):
+    first = max(0, pos - window + 1)
+    k, v = _cached(kcache, vcache, page_table, slot, first, pos + 1, page_size, 0)
+    seen = (pos - window + 1) // pool if pool and pos - window + 1 >= pool else 0
+    if seen:
+        pk, pv = _cached(kpool, vpool, page_table, slot, 0, seen, page_size, 0)
+        k, v = torch.cat([pk, k]), torch.cat([pv, v])
+    per = nh // nkv
+    out = torch.zeros(nh, dv, dtype=F64)
+    for h in range(nh):
+        s = (k[:, h // per, :].to(F64) @ q[h].to(F64)) * scale * (head_scale[h].to(F64) if head_scale is not None else 1.0)
+        out[h] = torch.softmax(s, dim=0) @ v[:, h // per, :].to(F64)
+    return out.reshape(-1)
+
+
+def attn_pooled_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, kpool, vpool, page_table, page_size,
+                     n_seqs, max_rows, nh, nkv, dk, dv, scale, head_scale, window, pool):
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+    for b in range(n_seqs):
+        s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+        for a in range(s1 - s0):
+            out[s0 + a] = _attend_pooled(q[s0 + a, :nh * dk].view(nh, dk), int(seq_start[b]) + a, int(seq_slot[b]),
+                                         kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv,
+                                         scale, head_scale, window, pool).to(q.dtype)
+    return out
+
+
+def attn_pooled_decode(q, kcache, vcache, kpool, vpool, page_table, page_size, seq_slot, seq_len, nh, nkv, dk,
+                       dv, scale, head_scale, window, pool):
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+    for b in range(q.shape[0]):
+        out[b] = _attend_pooled(q[b, :nh * dk].view(nh, dk), int(seq_len[b]) - 1, int(seq_slot[b]), kcache,
+                                vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, scale, head_scale,
+                                window, pool).to(q.dtype)
+    return out
+
+
+# ---------------------------------------------------------------- gated linear attention, a gated linear recurrent unit
+def gla_prepare(U, q_off, k_off, v_off, Z, z_bias, tau, H, dk, dv):
+    T = U.shape[0]
+    u = U.to(F64)
+    qn = (u[:, q_off:q_off + H * dk] * dk ** -0.5).view(T, H, dk)
+    kn = u[:, k_off:k_off + H * dk].view(T, H, dk)
+    vv = u[:, v_off:v_off + H * dv].view(T, H, dv)
+    z = Z.to(F64) + z_bias.to(F64)
+    dec = torch.exp(-_softplus(-z) / tau).view(T, H, dk)
+    beta = torch.ones(T, H, dtype=F64)
+    return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, beta, dec))
+
+
+def lru_gates(u, w_t, r_bias, i_bias, lam, rate):
+    T, C = u.shape
+    nb, cb = w_t.shape[1], w_t.shape[2]
+    ub = u.to(F64).view(T, nb, cb)
+    r = torch.sigmoid(torch.einsum("bio,tbi->tbo", w_t[0].to(F64), ub).reshape(T, C) + r_bias.to(F64))
+    i = torch.sigmoid(torch.einsum("bio,tbi->tbo", w_t[1].to(F64), ub).reshape(T, C) + i_bias.to(F64))
+    a = torch.exp(-rate * r * _softplus(lam.to(F64)))
+    x = torch.sqrt(torch.clamp(1 - a * a, min=0)) * i * u.to(F64)
+    return a.to(torch.float32), x.to(torch.float32)
+
+
+def lru_scan(a, x, state, Y, y_off, y_bias, cu_seqlens, seq_slot, n_seqs, out_dtype):
+    T, C = a.shape
+    out = torch.zeros(T, C, dtype=F64)
+    y = Y[:, y_off:y_off + C].to(F64) + (y_bias.to(F64) if y_bias is not None else 0.0)
+    y = 0.5 * y * (1 + torch.tanh(math.sqrt(2 / math.pi) * (y + 0.044715 * y ** 3)))
+    for b in range(n_seqs):
+        slot = int(seq_slot[b])
+        S = state[slot].to(F64)
+        for r in range(int(cu_seqlens[b]), int(cu_seqlens[b + 1])):
+            S = (a[r].to(F64) * S + x[r].to(F64)).to(torch.float32).to(F64)
+            out[r] = S * y[r]
+        state[slot] = S.to(torch.float32)
+    return out.to(out_dtype)
+
+
 def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
@@ -698,6 +870,8 @@ def patch(monkeypatch):
                  "few_outputs_f32", "moe_route", "moe_plan", "moe_experts", "moe_combine",
                  "stream_mix_norm", "kv_store2", "attn_cap_rows", "attn_cap_decode", "delta_prepare",
                  "delta_conv_tail", "delta_scan", "delta_finish", "qkv_norm_mix_store", "ssm_prepare",
-                 "ssm_finish", "memory_prepare", "memory_finish", "embed_pairs", "remember_last", "gelu_tanh"):
+                 "ssm_finish", "memory_prepare", "memory_finish", "embed_pairs", "remember_last", "gelu_tanh",
+                 "short_conv", "short_conv_tail", "rms_rows_gain", "clamped_swish_mul", "qk_rotate_store",
+                 "pool_store", "attn_pooled_rows", "attn_pooled_decode", "gla_prepare", "lru_gates", "lru_scan"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(ops.ScaledSum, "tensor", scaled_sum_tensor)
