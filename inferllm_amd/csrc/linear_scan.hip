@@ -327,9 +327,10 @@ lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, cons
         for (int r = 0; r < LRU_ROWS; ++r) {
             if (r >= rows) continue;
             const float rg = ls_sigmoid(ar[r] + b1), ig = ls_sigmoid(ai[r] + b2);
-            const float a = expf(-rate * rg * sp);
-            a_out[(size_t)(t0 + r) * C + c] = a;
-            x_out[(size_t)(t0 + r) * C + c] = sqrtf(fmaxf(1.0f - a * a, 0.f)) * ig * us[r * cb + o];
+            const float log_a = -rate * rg * sp;
+            a_out[(size_t)(t0 + r) * C + c] = expf(log_a);
+            // 1 - a^2 as -expm1(2 log a): a decay close to 1 keeps its digits
+            x_out[(size_t)(t0 + r) * C + c] = sqrtf(fmaxf(-expm1f(2.0f * log_a), 0.f)) * ig * us[r * cb + o];
         }
     }
 }
