@@ -22,13 +22,15 @@ of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
 The run fails (non-zero) if any timed run produced a non-finite logit or the same
 greedy token everywhere.
 
-`--design rabapel`, `--design kukupel` and `--design sabipel` are other workloads with a line of their own (the
+`--design rabapel`, `--design kukupel`, `--design sabipel` and `--design dotorax` are other workloads with a line of their own (the
 default's stays as it is):
 Rabapel (latent attention, layers that alternate a dense and a routed feed-forward) at two
 sizes beside LLaMA at the same width, heads and layer count: prefill of 2,048 tokens and decoding
 at batch 1, 8 and 64, each with its fraction of the matrix or HBM peak.
 Kukupel likewise beside Rabapel, and Sabipel (state-space, matrix-memory and chunked-attention
-layers with dense feed-forwards) beside Kukupel.
+layers with dense feed-forwards) beside Kukupel, and Dotorax (rotated attention with shared keys,
+gated linear attention, a window with pooled blocks beside a recurrent unit, gated feed-forwards,
+sublayers between two norms behind a short convolution) beside Sabipel.
 """
 import argparse
 import json
@@ -526,6 +528,121 @@ def sabipel_main(args) -> int:
     print(json.dumps(out), flush=True)
     return 0
 
+def dotorax_config(width, heads, kv_heads, layers, window=1024, pool=8, vocab=32000):
+    """Layers in the order attention, gla, parallel, attention that reads the first layer's keys ...:
+    attention heads of 128 query and 128 value dims with half of each head rotated, linear-attention
+    heads of 64 key and 128 value dims, a window of `window` tokens with blocks of `pool` beside a
+    recurrent unit as wide as the model in blocks of 128 or 256 channels, a gated feed-forward of
+    8/3 of the width in every layer, three taps in front of every sublayer."""
+    rot = {"base": 10000.0, "dims": 64}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "rot": rot}
+    gla = {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 16}
+    par = {"left": dict(att, mask={"size": window, "pool": pool}),
+           "right": {"width": width, "blocks": 16, "conv": 4}, "left_scale": 1.0, "right_scale": 1.0}
+    mlp = {"kind": "dense", "ff": 8 * width // 3 // 256 * 256, "limit": 7.0}
+    out = []
+    for i in range(layers):
+        kind = ("attention", "gla", "parallel", "attention")[i % 4]
+        mixer = dict(att) if kind == "attention" else dict(gla) if kind == "gla" else \
+            {k: (dict(v) if isinstance(v, dict) else v) for k, v in par.items()}
+        if i % 4 == 3:
+            mixer["kv_from"] = i - 3
+        out.append({"type": kind, "mixer": mixer, "mlp": dict(mlp)})
+    return {"architecture": "Dotorax", "vocab": vocab, "width": width, "max_positions": 8192,
+            "norm": {"eps": 1e-6}, "residual_mult": 0.5, "canon": {"taps": 3}, "layers": out}
+
+
+def dotorax_counts(cfg, esz):
+    """(step_bytes(batch, mean_ctx), flops(tokens, lens)) of a Dotorax configuration: the weights a
+    decode step reads, attention's cache rows (all of them, or a window's and the pooled rows before
+    it), the recurrent layers' float32 states (read and written); the multiply-adds of a prompt step
+    (attention over what each row sees, the linear attention's recurrence as 2 key x value products
+    a token and head, the recurrent unit's gates)."""
+    E, V = cfg["width"], cfg["vocab"]
+
+    def att_parts(m, own=True):
+        H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        return E * (H * dk + (G * (dk + dv) if own else 0)) + H * dv * E, G * (dk + dv), H * (dk + dv)
+
+    def layer_parts(layer):
+        """(weights, float32 state, cache columns a token, score columns a pair, window, pool, other multiply-adds a token)"""
+        m, kind = layer["mixer"], layer["type"]
+        ff = 3 * E * layer["mlp"]["ff"] if layer.get("mlp") else 0
+        if kind == "gla":
+            H, dk, dv, r = m["heads"], m["dim"], m["vdim"], m.get("rank", 16)
+            return E * (2 * H * dk + 2 * H * dv + r) + r * H * dk + H * dv * E + ff, H * dk * dv, 0, 0, 0, 0, 0
+        if kind == "attention":
+            w, kv, qk = att_parts(m, "kv_from" not in m)
+            return w + E * m["heads"] + ff, 0, kv, qk, 0, 0, 0
+        w, kv, qk = att_parts(m["left"])
+        C, nb = m["right"]["width"], m["right"]["blocks"]
+        gates = 2 * C * (C // nb)
+        return (w + 3 * E * C + gates + ff, C, kv, qk, m["left"]["mask"]["size"], m["left"]["mask"]["pool"], gates)
+
+    def seen(n, window, pool):
+        """keys that position n - 1 sees"""
+        if not window or n <= window:
+            return n
+        return window + (n - window) // pool
+
+    def step_bytes(batch, mean_ctx):
+        total = V * E * esz + batch * 3 * E * esz
+        for layer in cfg["layers"]:
+            w, state, kv_row, _, window, pool, _ = layer_parts(layer)
+            total += (w + batch * seen(int(mean_ctx), window, pool) * kv_row) * esz + batch * state * 4 * 2
+        return total
+
+    def flops(tokens, lens):
+        total = 2.0 * len(lens) * V * E
+        for layer in cfg["layers"]:
+            w, state, _, qk, window, pool, other = layer_parts(layer)
+            pairs = sum(sum(seen(p + 1, window, pool) for p in range(n)) for n in lens) if qk else 0
+            mem = 2 * state if layer["type"] == "gla" else 0
+            total += 2.0 * tokens * (w + other) + 2.0 * qk * pairs + 2.0 * mem * tokens
+        return total
+
+    return step_bytes, flops
+
+
+def dotorax_main(args) -> int:
+    """Dotorax at two sizes beside Sabipel, the library's closest design (recurrent layers with a
+    state per sequence, attention whose scores and weights stay float32), at the same width, heads
+    and number of layers (four): tokens/s of these four-layer models, with the fraction of the
+    matrix peak for prompts and of the HBM peak for decode steps."""
+    import torch
+    from inferllm_amd import Engine
+    layers = args.layers or 4
+    esz = 2 if args.dtype == "bfloat16" else 4
+    sizes = {"2048": dict(width=2048, heads=16, kv_heads=4), "4096": dict(width=4096, heads=32, kv_heads=8)}
+    few = min(args.steps, 128)
+    out = {"metric": "Dotorax beside Sabipel at equal width, heads and layers: prefill tok/s at 2,048 tokens, decode tok/s at batch 1/8/64",
+           "unit": "tokens/s", "n_gpus": 1, "steps": few, "warmup": 4, "dtype": "bf16" if esz == 2 else "fp32",
+           "data": "synthetic: seeded random weights, uniform random token ids", "layers": layers, "sizes": {}}
+    for name, sz in sizes.items():
+        if args.size and args.size != name:
+            continue
+        row = {}
+        dcfg = dotorax_config(layers=layers, **sz)
+        scfg = sabipel_config(layers=layers, **sz)
+        for design, cfg, counts in (("dotorax", dcfg, dotorax_counts), ("sabipel", scfg, sabipel_counts)):
+            if args.only and args.only != design:
+                continue
+            eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, device="cuda:0", max_batch=64,
+                                     max_seq_len=4096, max_tokens=64 * 1024)
+            b = Bench.around(eng, cfg["vocab"], layers, args.dtype, *counts(cfg, esz))
+            torch.cuda.synchronize()
+            r = {"prefill_2048": b.prefill_run(2048, reps=4)}
+            if not args.prefill_only:
+                for batch in (1, 8, 64):
+                    v, ms, f = b.decode_run(batch, few, 4, args.prompt)
+                    r[f"decode_b{batch}"] = {"value": round(v, 1), "ms": round(ms, 4), "hbm_frac": round(f, 4)}
+            row[design] = r
+            b.close()
+            del b, eng
+        out["sizes"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -544,12 +661,13 @@ def main() -> int:
     ap.add_argument("--no-70b", action="store_true",
                     help="leave the LLaMA-2-70B shape out of `points` (138 GB of weights: half a minute)")
     ap.add_argument("--with-70b", action="store_true", help="(the default now; kept for old command lines)")
-    ap.add_argument("--design", default="llama", choices=["llama", "rabapel", "kukupel", "sabipel"],
+    ap.add_argument("--design", default="llama", choices=["llama", "rabapel", "kukupel", "sabipel", "dotorax"],
                     help="rabapel: that design at two sizes beside LLaMA at equal size (a line of its own); "
                          "kukupel: that design at two sizes beside Rabapel at equal size (likewise); "
-                         "sabipel: that design at two sizes beside Kukupel at equal size (likewise)")
-    ap.add_argument("--size", default="", help="with --design rabapel, kukupel or sabipel: only this width (2048 or 4096)")
-    ap.add_argument("--only", default="", help="with --design kukupel or sabipel: only this one of the two designs")
+                         "sabipel: that design at two sizes beside Kukupel at equal size (likewise); "
+                         "dotorax: that design at two sizes beside Sabipel at equal size (likewise)")
+    ap.add_argument("--size", default="", help="with --design rabapel, kukupel, sabipel or dotorax: only this width (2048 or 4096)")
+    ap.add_argument("--only", default="", help="with --design kukupel, sabipel or dotorax: only this one of the two designs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
@@ -561,6 +679,8 @@ def main() -> int:
         return kukupel_main(args)
     if args.design == "sabipel":
         return sabipel_main(args)
+    if args.design == "dotorax":
+        return dotorax_main(args)
 
     shape_name, shape_cfg = SHAPES[args.shape]
     ctx_len = shape_cfg["max_position_embeddings"]

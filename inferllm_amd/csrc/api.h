@@ -480,6 +480,14 @@ int illm_short_conv_tail(const void* X, int x_dt, int x_stride, int x_off, const
 // out[r] = gain * a[r] / sqrt(mean(a[r]^2) + eps) * w, float32.
 int illm_rms_rows_gain(const void* a, int a_dt, const void* w, int w_dt, float* out, int rows, int E,
                        float eps, float gain, void* stream);
+// x <- x + gain * a / sqrt(mean(a^2) + post_eps) * post_w (a null: nothing added); h = rmsnorm(x, eps) * w
+// in the output's type; out = h + conv over time with the earlier inputs from tail [slots, taps - 1, E],
+// which is moved on (conv_w null: out = h; the convolution is for steps of one row a sequence).  With
+// row_idx only those rows are formed and x stays.  E floats of LDS: E <= 16384.
+int illm_post_add_rmsnorm(float* x, const void* a, int a_dt, const void* post_w, int post_w_dt,
+                          float post_eps, float gain, const void* w, int w_dt, void* out, int out_dt,
+                          const int32_t* row_idx, int rows, int E, float eps, const float* conv_w,
+                          int taps, void* tail, int tail_dt, const int32_t* row_slot, void* stream);
 // gate_up [T, 2F]: out = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
 int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, int T, int F, float limit,
                            float alpha, void* stream);

@@ -164,3 +164,94 @@ extern "C" int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, in
     }
     return illm_launch_status();
 }
+
+// ---------------------------------------------------------------- one pass between two sublayers
+// What stands between a sublayer that has its own norm behind it and the next sublayer's input:
+//     x <- x + gain * a / sqrt(mean(a^2) + post_eps) * post_w          (a null: nothing is added)
+//     h  = x / sqrt(mean(x^2) + eps) * w                                (rounded to the output's type)
+//     out = h + sum_j conv_w[:, j] h(t - (taps - 1 - j))                (conv_w null: out = h)
+// With `row_idx` only those rows are formed and x is left as it is.  The convolution is for steps of
+// one row a sequence: the earlier inputs come from tail [slots][taps - 1][E], which is moved on.
+// grid (rows); 256 threads; the row's sum is kept in LDS (E floats) between the passes.
+__global__ void __launch_bounds__(256)
+post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a_dt,
+                        const void* __restrict__ post_w, int post_w_dt, float post_eps, float gain,
+                        const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
+                        const int32_t* __restrict__ row_idx, int E, float eps,
+                        const float* __restrict__ conv_w, int taps, void* __restrict__ tail, int tail_dt,
+                        const int32_t* __restrict__ row_slot) {
+    extern __shared__ float row[];
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int in_row = row_idx ? row_idx[r] : r;
+    const size_t ib = (size_t)in_row * E, ob = (size_t)r * E;
+    float inv_a = 0.f;
+    if (a) {
+        float sa = 0.f;
+        for (int i = threadIdx.x; i < E; i += 256) {
+            const float v = ld_f(a, a_dt, ib + i);
+            sa = fmaf(v, v, sa);
+        }
+        sa = block_sum(sa, red);
+        inv_a = 1.0f / sqrtf(sa / (float)E + post_eps);
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < E; i += 256) {
+        float v = x[ib + i];
+        if (a) {
+            v += gain * (ld_f(a, a_dt, ib + i) * inv_a * ld_f(post_w, post_w_dt, i));
+            if (!row_idx) x[ib + i] = v;
+        }
+        row[i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)E + eps);
+    const int K = taps - 1;
+    const int slot = conv_w ? row_slot[r] : 0;
+    for (int i = threadIdx.x; i < E; i += 256) {
+        float h = (row[i] * scale) * ld_f(w, w_dt, i);
+        if (conv_w) {
+            h = conv_round(h, out_dt);
+            float y = h;
+            float in[CONV_MAX_TAPS];
+#pragma unroll
+            for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+                if (j >= taps) continue;
+                in[j] = j == K ? h : ld_f(tail, tail_dt, ((size_t)slot * K + j) * E + i);
+            }
+            float c = 0.f;
+#pragma unroll
+            for (int j = 0; j < CONV_MAX_TAPS; ++j)
+                if (j < taps) c = fmaf(conv_w[(size_t)i * taps + j], in[j], c);
+            y += c;
+#pragma unroll
+            for (int j = 1; j < CONV_MAX_TAPS; ++j)
+                if (j < taps) st_f(tail, tail_dt, ((size_t)slot * K + (j - 1)) * E + i, in[j]);
+            h = y;
+        }
+        st_f(out, out_dt, ob + i, h);
+    }
+}
+
+extern "C" int illm_post_add_rmsnorm(float* x, const void* a, int a_dt, const void* post_w, int post_w_dt,
+                                     float post_eps, float gain, const void* w, int w_dt, void* out,
+                                     int out_dt, const int32_t* row_idx, int rows, int E, float eps,
+                                     const float* conv_w, int taps, void* tail, int tail_dt,
+                                     const int32_t* row_slot, void* stream) {
+    if (rows < 0 || E <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
+        (a && (!illm_dtype_ok(a_dt) || !illm_dtype_ok(post_w_dt) || !post_w)) ||
+        (conv_w && (taps < 2 || taps > CONV_MAX_TAPS || !tail || !row_slot || row_idx || !illm_dtype_ok(tail_dt))))
+        return ILLM_ERR_ARG;
+    if (rows == 0) return ILLM_OK;
+    const size_t lds = (size_t)E * sizeof(float);
+    if (lds > 64 * 1024) return ILLM_ERR_ARG;
+    if (lds > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)post_add_rmsnorm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+        return ILLM_ERR_LAUNCH;
+    hipLaunchKernelGGL(post_add_rmsnorm_kernel, dim3(rows), dim3(256), lds, (hipStream_t)stream, x, a, a_dt,
+                       post_w, post_w_dt, post_eps, gain, w, w_dt, out, out_dt, row_idx, E, eps, conv_w, taps,
+                       tail, tail_dt, row_slot);
+    return illm_launch_status();
+}

@@ -1854,6 +1854,56 @@ def rms_rows_gain(a: torch.Tensor, weight: torch.Tensor, eps: float, gain: float
     return out
 
 
+class PostNormed:
+    """gain * a / sqrt(mean(a^2) + eps) * weight, not yet formed: what a sublayer with a norm of its
+    own behind it leaves to be added to the residual stream.  A norm that adds it in its own kernel
+    (`post_add_rmsnorm`) takes the pieces, any other asks for `tensor()` (float32)."""
+
+    def __init__(self, a: torch.Tensor, weight: torch.Tensor, eps: float, gain: float):
+        self.a, self.weight, self.eps, self.gain = a, weight, float(eps), float(gain)
+
+    def tensor(self) -> torch.Tensor:
+        return rms_rows_gain(self.a, self.weight, self.eps, self.gain)
+
+
+POST_ADD_MAX_WIDTH = 16384
+
+
+def post_add_rmsnorm(x: torch.Tensor, post: Optional[PostNormed], weight: torch.Tensor, eps: float,
+                     out_dtype: torch.dtype, row_idx: Optional[torch.Tensor] = None, conv=None) -> torch.Tensor:
+    """One pass between two sublayers: x += `post` (its norm formed here; None: nothing), then the
+    RMS norm of x under `weight` in `out_dtype`, then, with `conv` = (weight float32 [E, taps], tail
+    [slots, taps - 1, E], row_slot), the normed row plus its short convolution over time, the tail
+    moved on (for steps of one row a sequence).  With `row_idx` only those rows, and x stays."""
+    _gpu(x, weight, row_idx)
+    _i32(row_idx)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "post_add_rmsnorm: x must be float32 [T, E]")
+    T, E = x.shape
+    _need(weight.shape == (E,) and E <= POST_ADD_MAX_WIDTH, f"post_add_rmsnorm: weight [{E}], width up to {POST_ADD_MAX_WIDTH}")
+    a = pw = None
+    if post is not None:
+        a, pw = post.a, post.weight
+        _gpu(a, pw)
+        _need(a.shape == x.shape and pw.shape == (E,), "post_add_rmsnorm: the sublayer's output has x's shape")
+    rows = T if row_idx is None else row_idx.numel()
+    cw = tail = slots = None
+    taps = 0
+    if conv is not None:
+        cw, tail, slots = conv
+        _gpu(cw, tail, slots)
+        _i32(slots, T)
+        taps = cw.shape[1]
+        _need(row_idx is None and cw.dtype == torch.float32 and cw.shape == (E, taps) and 2 <= taps <= 8
+              and tail.dim() == 3 and tail.shape[1:] == (taps - 1, E), "post_add_rmsnorm: convolution shapes")
+    out = torch.empty((rows, E), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_post_add_rmsnorm(
+        _p(x), _p(a), _code(a) if a is not None else 0, _p(pw), _code(pw) if pw is not None else 0,
+        ctypes.c_float(post.eps if post is not None else 0.0), ctypes.c_float(post.gain if post is not None else 0.0),
+        _p(weight), _code(weight), _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _p(cw), taps,
+        _p(tail), _code(tail) if tail is not None else 0, _p(slots), _stream()), "post_add_rmsnorm")
+    return out
+
+
 SWISH_ALPHA = 1.702
 
 

@@ -107,6 +107,9 @@ class SandwichBlock(Block):
 
     graph_safe_prompts = True
 
+    takes_next_norm = True           # to hand a norm that forms a sublayer's own norm the pieces
+    takes_prepared_rows = True       # (prepared rows mean: the sum is in x already)
+
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, position, size: int,
                  eps: float, gain: float = 1.0, taps: int = 0, weight_offset: float = 0.0, tensors=None):
         super().__init__(mixer, feed_forward, mixer_norm, feed_forward_norm, position, tensors)
@@ -142,28 +145,48 @@ class SandwichBlock(Block):
             if self.taps:
                 self.conv[q - 1] = self._take(tensors, f"conv{q}").to(torch.float32).contiguous()
 
+    def _tail(self, q: int, ctx: StepContext):
+        return ctx.cache.state_line(("block", ctx.run))[f"tail{q}"]
+
     def _read(self, h, q: int, ctx: StepContext):
         """What sublayer q reads: the normed rows plus their convolution over time."""
         if not self.taps:
             return h
-        if self.taps == 1:
-            tail = h.new_zeros((1, 1, self.size))
-        else:
-            tail = ctx.cache.state_line(("block", ctx.run))[f"tail{q}"]
+        tail = self._tail(q, ctx) if self.taps > 1 else h.new_zeros((1, 1, self.size))
         out = ops.short_conv(h, 0, self.size, self.conv[q - 1], tail, ctx.row_slot, h.dtype,
                              add_input=True, update_tail=not ctx.prefill)
         if ctx.prefill and self.taps > 1:
             ops.short_conv_tail(h, 0, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps)
         return out
 
-    def forward(self, x, pending, ctx: StepContext, line, writes_cache):
-        h = self._read(self.mixer_norm.forward(x, pending, ctx), 1, ctx)
+    def _enter(self, norm, q: int, x, pending, ctx: StepContext):
+        """Sublayer q's input: `pending` added to x, the norm, the convolution.  A plain RMS norm
+        and a step of single tokens make that one kernel."""
+        if isinstance(pending, ops.NormedRows):
+            pending = None                       # its sum is in x already
+        params = norm.rms_params()
+        plain = pending is None or isinstance(pending, ops.PostNormed)
+        if (params is not None and plain and not ctx.prefill and self.taps > 1
+                and self.size <= ops.POST_ADD_MAX_WIDTH):
+            return ops.post_add_rmsnorm(x, pending, params[0], params[1], ctx.act_dtype,
+                                        conv=(self.conv[q - 1], self._tail(q, ctx), ctx.row_slot))
+        if isinstance(pending, ops.PostNormed) and not getattr(norm, "adds_post_normed", False):
+            pending = pending.tensor()
+        return self._read(norm.forward(x, pending, ctx), q, ctx)
+
+    def _leave(self, y, q: int, next_norm):
+        """What sublayer q leaves to be added: its output under its own norm, times the gain; as
+        pieces if the norm that follows forms them in its own pass."""
+        post = ops.PostNormed(y, self.post[q - 1], self.eps, self.gain)
+        return post if next_norm is not None and getattr(next_norm, "adds_post_normed", False) else post.tensor()
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache, next_norm=None):
+        h = self._enter(self.mixer_norm, 1, x, pending, ctx)
         a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
-        d = ops.rms_rows_gain(a, self.post[0], self.eps, self.gain)
         if not self.has_ff:
-            return d
-        h2 = self._read(self.feed_forward_norm.forward(x, d, ctx), 2, ctx)
-        return ops.rms_rows_gain(self.feed_forward.forward(h2, ctx), self.post[1], self.eps, self.gain)
+            return self._leave(a, 1, next_norm)
+        h2 = self._enter(self.feed_forward_norm, 2, x, self._leave(a, 1, self.feed_forward_norm), ctx)
+        return self._leave(self.feed_forward.forward(h2, ctx), 2, next_norm)
 
 
 @register_part("block", "hyper_connections")

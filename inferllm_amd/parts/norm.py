@@ -44,7 +44,15 @@ class RMSNorm(Norm):
     def rms_params(self):
         return self.weight, self.eps
 
+    # `forward` also takes `delta` as `ops.PostNormed` (a sublayer's output whose own norm is still
+    # to be formed) and forms it in the same pass
+    adds_post_normed = True
+
     def forward(self, x, delta, ctx: StepContext, row_idx=None):
+        if isinstance(delta, ops.PostNormed):
+            if self.size <= ops.POST_ADD_MAX_WIDTH:
+                return ops.post_add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, row_idx)
+            delta = delta.tensor()
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, row_idx)
 
     def forward_with(self, other: "RMSNorm", x, delta, ctx: StepContext):

@@ -740,6 +740,15 @@ def rms_rows_gain(a, weight, eps, gain):
     return (gain * (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(F64))).to(torch.float32)
 
 
+def post_add_rmsnorm(x, post, weight, eps, out_dtype, row_idx=None, conv=None):
+    delta = rms_rows_gain(post.a, post.weight, post.eps, post.gain) if post is not None else None
+    h = add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx)
+    if conv is None:
+        return h
+    cw, tail, slots = conv
+    return short_conv(h, 0, h.shape[1], cw, tail, slots, out_dtype, add_input=True, update_tail=True)
+
+
 def clamped_swish_mul(gate_up, limit):
     F = gate_up.shape[1] // 2
     g = torch.clamp(gate_up[:, :F].to(F64), max=limit)
@@ -871,7 +880,7 @@ def patch(monkeypatch):
                  "stream_mix_norm", "kv_store2", "attn_cap_rows", "attn_cap_decode", "delta_prepare",
                  "delta_conv_tail", "delta_scan", "delta_finish", "qkv_norm_mix_store", "ssm_prepare",
                  "ssm_finish", "memory_prepare", "memory_finish", "embed_pairs", "remember_last", "gelu_tanh",
-                 "short_conv", "short_conv_tail", "rms_rows_gain", "clamped_swish_mul", "qk_rotate_store",
+                 "short_conv", "short_conv_tail", "rms_rows_gain", "post_add_rmsnorm", "clamped_swish_mul", "qk_rotate_store",
                  "pool_store", "attn_pooled_rows", "attn_pooled_decode", "gla_prepare", "lru_gates", "lru_scan"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(ops.ScaledSum, "tensor", scaled_sum_tensor)

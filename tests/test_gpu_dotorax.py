@@ -471,6 +471,21 @@ def test_norm_with_a_gain_and_clamped_gate_against_plain_torch(dtype):
         _near(ops.rms_rows_gain(a.cuda(), w.cuda(), 1e-5, 0.3), R.rms_rows_gain(a, w, 1e-5, 0.3), 1e-5)
         gu = (torch.randn(T, 2 * E, generator=g) * 2).to(dtype)
         _near(ops.clamped_swish_mul(gu.cuda(), 1.25), R.clamped_swish_mul(gu, 1.25), tol)
+        # the pass between two sublayers: the sublayer's own norm, the add, the next norm, and for
+        # single tokens the convolution with its tail; or only some rows, with x left as it is
+        x, w2 = torch.randn(T, E, generator=g), (torch.randn(E, generator=g) + 1).to(dtype)
+        cw, tail = torch.randn(E, 3, generator=g), torch.randn(T + 1, 2, E, generator=g).to(dtype)
+        slots = torch.randperm(T, generator=g).to(torch.int32)
+        idx = torch.tensor([T - 1, 0], dtype=torch.int32)
+        for post in (None, (a, w, 1e-5, 0.3)):
+            for conv, rows in ((None, None), (None, idx), ((cw, tail, slots), None)):
+                x_want, x_got, t_want, t_got = x.clone(), x.cuda(), tail.clone(), tail.cuda()
+                want = R.post_add_rmsnorm(x_want, ops.PostNormed(*post) if post else None, w2, 2e-5, dtype, rows,
+                                          (cw, t_want, slots) if conv else None)
+                got = ops.post_add_rmsnorm(x_got, ops.PostNormed(a.cuda(), w.cuda(), 1e-5, 0.3) if post else None,
+                                           w2.cuda(), 2e-5, dtype, rows.cuda() if rows is not None else None,
+                                           (cw.cuda(), t_got, slots.cuda()) if conv else None)
+                _near(got, want, tol); _near(x_got, x_want, 1e-5); _near(t_got, t_want, tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
