@@ -411,16 +411,18 @@ int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int
                        const void* vcache, const int32_t* page_table, int table_stride,
                        int page_size, int ring, int n_seqs, int max_rows, int nh, int nkv, int dk,
                        int dv, float scale, float cap, int window, const float* slopes, int chunk,
-                       const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream);
+                       const void* gate, int gate_stride, int gate_off, int gate_heads, float* lse, void* stream);
 int illm_attn_cap_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
                          const void* vcache, const int32_t* page_table, int table_stride,
                          int page_size, int ring, const int32_t* seq_slot, const int32_t* seq_len,
                          float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
                          float scale, float cap, int window, const float* slopes, int chunk,
-                         const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream);
+                         const void* gate, int gate_stride, int gate_off, int gate_heads, float* lse, void* stream);
 // The two calls above also take: `slopes` float32 [nh] (null: none), score -= slopes[h] (i - j);
 // `chunk` > 0, a row sees only the keys j with floor(j / chunk) = floor(i / chunk); `gate` (null: none),
-// rows [., gate_stride] of the queries' dtype, out *= sigmoid(gate[row, gate_off + h dv + d]).
+// rows [., gate_stride] of the queries' dtype, out *= sigmoid(gate[row, gate_off + h dv + d]) (with
+// `gate_heads` gate[row, gate_off + h]); `lse` (null: none), float32 [rows, nh]: max + log(sum) of each
+// softmax (single tokens: with nsplit >= 2).
 // In place: q and k of rows [q (nh dk) | .. k at k_off | v at v_off] each divided by the root mean
 // square over all their heads and multiplied by qw, kw (null: untouched); v <- (1 - lam[0]) v +
 // lam[0] first[row, first_off ..] (lam null: untouched); k and v stored in the paged cache (null: not).
@@ -495,11 +497,12 @@ int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, int T, int F,
 // ---- attention over a window of tokens and pooled blocks before it (attention_pooled.hip)
 // In place on packed rows [q (nh dk) | .. k at k_off (nkv dk) | v at v_off (nkv dv)]: q and k heads
 // turned by their positions (cos_sin float32 [n_positions, rot / 2, 2]; pairing 0: i with i + rot / 2,
-// 1: 2i with 2i + 1; null: none), then, with `unit_norm`, divided by their root mean square; k and v
+// 1: 2i with 2i + 1; null: none), then, with `unit_norm`, divided by their root mean square, query head
+// h then times q_scale[h] (float32 [nh]; null: none); k and v
 // stored in the paged cache (kcache null: not stored; nkv 0: queries alone).
 int illm_qk_rotate_store(void* rows, int dt, int row_len, int k_off, int v_off, const float* cos_sin,
                          int rot, int pairing, int n_positions, int unit_norm, float eps,
-                         const int32_t* row_pos, const int32_t* row_slot, void* kcache, void* vcache,
+                         const float* q_scale, const int32_t* row_pos, const int32_t* row_slot, void* kcache, void* vcache,
                          const int32_t* page_table, int table_stride, int page_size, int ring, int T,
                          int nh, int nkv, int dk, int dv, void* stream);
 // For every row whose position ends a block of `pool` tokens: the block's mean key and value, from
@@ -515,14 +518,16 @@ int illm_attn_pooled_rows(const void* q, int q_stride, void* out, int dt, const 
                           const void* vcache, const void* kpool, const void* vpool,
                           const int32_t* page_table, int table_stride, int page_size, int n_seqs,
                           int max_rows, int nh, int nkv, int dk, int dv, float scale,
-                          const float* head_scale, int window, int pool, void* stream);
+                          const float* head_scale, int window, int pool, const float* lse, void* stream);
+// With `lse` (float32 [rows, nh]) the tokens of the window are done already: `out` holds their
+// normalised sums and `lse` max + log(sum) of their softmax, and the pooled rows are merged in place.
 // The same for one new token a sequence, at position seq_len - 1.
 int illm_attn_pooled_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
                             const void* vcache, const void* kpool, const void* vpool,
                             const int32_t* page_table, int table_stride, int page_size,
                             const int32_t* seq_slot, const int32_t* seq_len, int B, int nh, int nkv,
                             int dk, int dv, float scale, const float* head_scale, int window, int pool,
-                            void* stream);
+                            const float* lse, void* stream);
 
 // ---- gated linear attention and a gated linear recurrent unit (linear_scan.hip)
 // Inputs of the plain gated rule with a decay per key channel: q dk^-1/2, k, v from U; decay =
@@ -536,10 +541,11 @@ int illm_gla_prepare(const void* U, int dt, int u_stride, int q_off, int k_off, 
 int illm_lru_gates(const float* u, const float* Wt, const float* br, const float* bi, const float* lam,
                    float rate, float* a_out, float* x_out, int T, int C, int nb, void* stream);
 // S <- a S + x per channel over every sequence's rows from state [slots, C] and back into it;
-// out = S gelu_tanh(Y[:, y_off + c] + yb[c]).
+// out = S gelu_tanh(Y[:, y_off + c] + yb[c]).  `scratch` (may be null): 2 n_seqs ceil(max_rows / 32) C
+// floats, with which steps of 64 rows a sequence or more run chunk by chunk in parallel.
 int illm_lru_scan(const float* a, const float* x, float* state, const void* Y, int y_dt, int y_stride,
                   int y_off, const float* yb, void* out, int out_dt, const int32_t* cu,
-                  const int32_t* seq_slot, int n_seqs, int C, void* stream);
+                  const int32_t* seq_slot, int n_seqs, int max_rows, int C, float* scratch, void* stream);
 
 #ifdef __cplusplus
 }

@@ -5,7 +5,9 @@
 // a bias by distance, score -= slopes[h] (i - j) (`slopes` null: none); chunks, position i sees only
 // the keys of its own chunk, floor(j / chunk) = floor(i / chunk), counted from the sequence's
 // position 0 (`chunk` <= 0: none); an output gate, out *= sigmoid(gate[row, gate_off + h dv + d])
-// (`gate` null: none; with `gate_heads` one number a head, gate[row, gate_off + h]).  Positions enter through the bias and the chunks alone.
+// (`gate` null: none; with `gate_heads` one number a head, gate[row, gate_off + h]).  Positions enter
+// through the bias and the chunks alone.  `lse` (null: none) takes max + log(sum) of every row's and
+// head's softmax, [rows][heads], for whoever goes on with further keys.
 // Keys and values live in the paged cache, K [page][kv head][row][dk], V [page][kv head][row][dv],
 // under one page table; a step first stores its rows (`kv_store2`) and then every row attends over
 // the cache at absolute positions, so whole prompts, portions of prompts and single tokens take
@@ -153,7 +155,8 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
                      const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                      int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
                      float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
-                     const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads) {
+                     const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads,
+                     float* __restrict__ lse) {
     extern __shared__ float smem[];
     const int kp = dk + 1, vp = dv + 1;
     float* qs = smem;               // [CQ][kp]
@@ -242,6 +245,7 @@ attn_cap_rows_kernel(const void* __restrict__ q, int q_stride, void* __restrict_
     }
     if (qrow < len) {
         const float inv = 1.0f / l_i;
+        if (lse && g == 0) lse[(size_t)(start + qrow) * nh + h] = m_i + logf(l_i);
         const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
         const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * (gate_heads ? 1 : dv);
 #pragma unroll
@@ -313,7 +317,8 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
                           const void* __restrict__ vcache, const int32_t* __restrict__ page_table,
                           int table_stride, int page_size, int ring, int nh, int nkv, int dk, int dv,
                           float scale, float cap, int window, const float* __restrict__ slopes, int chunk,
-                          const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads) {
+                          const void* __restrict__ gate, int gate_stride, int gate_off, int gate_heads,
+                          float* __restrict__ lse) {
     constexpr int DKP = 32 * KT, DVP = 32 * VT, KLD = DKP + 1;
     __shared__ float ks[MK * KLD];
     __shared__ float vs[MK * DVP];
@@ -441,6 +446,7 @@ attn_cap_rows_mfma_kernel(const void* __restrict__ q, int q_stride, void* __rest
     }
     if (qrow < len) {
         const float inv = 1.0f / l_i;
+        if (lse && half == 0) lse[(size_t)(start + qrow) * nh + h] = m_i + logf(l_i);
         const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
         const size_t gb = (size_t)(start + qrow) * gate_stride + gate_off + (size_t)h * (gate_heads ? 1 : dv);
 #pragma unroll
@@ -468,7 +474,7 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
                                   int table_stride, int page_size, int ring, int n_seqs, int max_rows,
                                   int nh, int nkv, int dk, int dv, float scale, float cap, int window,
                                   const float* slopes, int chunk, const void* gate, int gate_stride,
-                                  int gate_off, int gate_heads, void* stream) {
+                                  int gate_off, int gate_heads, float* lse, void* stream) {
     if (gate && (gate_off < 0 || gate_off + nh * (gate_heads ? 1 : dv) > gate_stride)) return ILLM_ERR_ARG;
     if (n_seqs < 0 || max_rows < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 ||
         dv <= 0 || dv > 256 || page_size <= 0 || !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
@@ -480,7 +486,7 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
 #define GO(DT_, KT_, VT_)                                                                          \
     hipLaunchKernelGGL((attn_cap_rows_mfma_kernel<DT_, KT_, VT_>), grid, dim3(256), 0, (hipStream_t)stream, \
                        q, q_stride, out, cu, seq_slot, seq_start, kcache, vcache, page_table, table_stride, \
-                       page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, gate, gate_stride, gate_off, gate_heads)
+                       page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes, chunk, gate, gate_stride, gate_off, gate_heads, lse)
 #define GO_V(DT_, KT_)                                                                             \
     switch (vt) { case 1: GO(DT_, KT_, 1); break; case 2: GO(DT_, KT_, 2); break;                  \
                   case 3: GO(DT_, KT_, 3); break; default: GO(DT_, KT_, 4); break; }
@@ -501,7 +507,7 @@ extern "C" int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt
     hipLaunchKernelGGL(attn_cap_rows_kernel, dim3((max_rows + CQ - 1) / CQ, nh, n_seqs), dim3(256), lds,
                        (hipStream_t)stream, q, q_stride, out, dt, cu, seq_slot, seq_start, kcache, vcache,
                        page_table, table_stride, page_size, ring, nh, nkv, dk, dv, scale, cap, window, slopes,
-                       chunk, gate, gate_stride, gate_off, gate_heads);
+                       chunk, gate, gate_stride, gate_off, gate_heads, lse);
     return illm_launch_status();
 }
 
@@ -809,7 +815,7 @@ attn_cap_decode_rows8_kernel(const void* __restrict__ q, int q_stride, const voi
 // grid (heads, sequences): combine the splits' partial results in split order.
 __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* __restrict__ out,
                                       int dt, int nsplit, int nh, int dv, const void* __restrict__ gate,
-                                      int gate_stride, int gate_off, int gate_heads) {
+                                      int gate_stride, int gate_off, int gate_heads, float* __restrict__ lse) {
     const int h = blockIdx.x, b = blockIdx.y;
     const float* pp = partial + ((size_t)b * nh + h) * nsplit * (dv + 2);
     float mm = NEG_INF;
@@ -820,6 +826,7 @@ __global__ void attn_cap_merge_kernel(const float* __restrict__ partial, void* _
         lt += (ms == NEG_INF ? 0.f : expf(ms - mm)) * pp[(size_t)s * (dv + 2) + dv + 1];
     }
     const float inv = 1.0f / lt;
+    if (lse && threadIdx.x == 0) lse[(size_t)b * nh + h] = mm + logf(lt);
     for (int d = threadIdx.x; d < dv; d += blockDim.x) {
         float a = 0.f;
         for (int s = 0; s < nsplit; ++s) {
@@ -838,10 +845,11 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
                                     int ring, const int32_t* seq_slot, const int32_t* seq_len,
                                     float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
                                     float scale, float cap, int window, const float* slopes, int chunk,
-                                    const void* gate, int gate_stride, int gate_off, int gate_heads, void* stream) {
+                                    const void* gate, int gate_stride, int gate_off, int gate_heads, float* lse, void* stream) {
     if (gate && (gate_off < 0 || gate_off + nh * (gate_heads ? 1 : dv) > gate_stride)) return ILLM_ERR_ARG;
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 ||
-        page_size <= 0 || nsplit < 1 || nsplit > 65535 || B > 65535 || !illm_dtype_ok(dt) || !partial)
+        page_size <= 0 || nsplit < 1 || nsplit > 65535 || B > 65535 || !illm_dtype_ok(dt) || !partial ||
+        (lse && nsplit < 2))                       // the kernel that merges the ranges writes it
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
@@ -882,6 +890,6 @@ extern "C" int illm_attn_cap_decode(const void* q, int q_stride, void* out, int 
                            seq_len, partial, nsplit, nh, nkv, dk, dv, scale, cap, window, slopes, chunk);
     if (hipGetLastError() != hipSuccess) return ILLM_ERR_LAUNCH;
     hipLaunchKernelGGL(attn_cap_merge_kernel, dim3(nh, B), dim3(64), 0, st, partial, out, dt, nsplit, nh, dv,
-                       gate, gate_stride, gate_off, gate_heads);
+                       gate, gate_stride, gate_off, gate_heads, lse);
     return illm_launch_status();
 }

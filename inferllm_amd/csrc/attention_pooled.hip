@@ -6,11 +6,16 @@
 // The pooled rows live in the same paged cache line as the tokens, under the same page table: block
 // b is row b of the sequence ("kp", "vp" beside "k", "v"), so it is there as soon as its last token
 // is and is read densely.  score = (q . k) scale head_scale[h] (`head_scale` null: 1).
+// The attention kernels do both parts themselves, or, given `lse`, the pooled part alone on top of
+// what a kernel for windows left: `out` holds the window's normalised sums and `lse` [rows][heads]
+// max + log(sum) of its softmax (attention_capped.hip writes both), and the pooled rows are merged
+// into `out` in place.
 // Float32 arithmetic over float32 or bfloat16 storage; key and value widths of up to 256.
 //
 // Beside the attention: `qk_rotate_store` turns q and k of packed rows by their positions (either
-// pairing, the first `rot` dims of a head), optionally divides every head by its root mean square,
-// and stores k and v (widths of their own) in the cache; `pool_store` forms the pooled rows of the
+// pairing, the first `rot` dims of a head), optionally divides every head by its root mean square
+// and multiplies query head h by q_scale[h] (a scale of the scores that differs by head, taken into
+// the queries), and stores k and v (widths of their own) in the cache; `pool_store` forms the pooled rows of the
 // blocks that a step completes.
 #include <math.h>
 
@@ -27,7 +32,7 @@
 __global__ void __launch_bounds__(64)
 qk_rotate_store_kernel(void* __restrict__ rows, int dt, int row_len, int k_off, int v_off,
                        const float* __restrict__ cos_sin, int rot, int pairing, int unit_norm, float eps,
-                       const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                       const float* __restrict__ q_scale, const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
                        void* __restrict__ kcache, void* __restrict__ vcache,
                        const int32_t* __restrict__ page_table, int table_stride, int page_size, int ring,
                        int nh, int nkv, int dk, int dv) {
@@ -57,6 +62,7 @@ qk_rotate_store_kernel(void* __restrict__ rows, int dt, int row_len, int k_off, 
         ss = wave_sum(ss);
         inv = 1.0f / sqrtf(ss / (float)dk + eps);
     }
+    if (q_scale && !is_k) inv *= q_scale[h];
     size_t kat = 0, vat = 0;
     const bool store = is_k && kcache != nullptr;
     if (store) {
@@ -80,7 +86,7 @@ qk_rotate_store_kernel(void* __restrict__ rows, int dt, int row_len, int k_off, 
 
 extern "C" int illm_qk_rotate_store(void* rows, int dt, int row_len, int k_off, int v_off,
                                     const float* cos_sin, int rot, int pairing, int n_positions,
-                                    int unit_norm, float eps, const int32_t* row_pos,
+                                    int unit_norm, float eps, const float* q_scale, const int32_t* row_pos,
                                     const int32_t* row_slot, void* kcache, void* vcache,
                                     const int32_t* page_table, int table_stride, int page_size, int ring,
                                     int T, int nh, int nkv, int dk, int dv, void* stream) {
@@ -91,7 +97,7 @@ extern "C" int illm_qk_rotate_store(void* rows, int dt, int row_len, int k_off, 
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
     hipLaunchKernelGGL(qk_rotate_store_kernel, dim3(T, nh + nkv), dim3(64), 0, (hipStream_t)stream, rows,
-                       dt, row_len, k_off, v_off, cos_sin, rot, pairing, unit_norm, eps, row_pos, row_slot,
+                       dt, row_len, k_off, v_off, cos_sin, rot, pairing, unit_norm, eps, q_scale, row_pos, row_slot,
                        kcache, vcache, page_table, table_stride, page_size, ring, nh, nkv, dk, dv);
     return illm_launch_status();
 }
@@ -156,7 +162,8 @@ attn_pooled_rows_kernel(const void* __restrict__ q, int q_stride, void* __restri
                         const void* __restrict__ vcache, const void* __restrict__ kpool,
                         const void* __restrict__ vpool, const int32_t* __restrict__ page_table,
                         int table_stride, int page_size, int nh, int nkv, int dk, int dv, float scale,
-                        const float* __restrict__ head_scale, int window, int pool) {
+                        const float* __restrict__ head_scale, int window, int pool,
+                        const float* __restrict__ lse) {
     extern __shared__ float smem[];
     const int kp = dk + 1, vp = dv + 1;
     float* qs = smem;               // [PQ][kp]
@@ -184,8 +191,23 @@ attn_pooled_rows_kernel(const void* __restrict__ q, int q_stride, void* __restri
     const int qrow = q0 + i, qpos = pos0 + qrow;
     const int last_pos = min(total, pos0 + q0 + PQ) - 1;
     const int seen_i = pool > 0 ? blocks_seen(qpos, window, pool) : 0;
+    if (lse) {
+        // the tokens of the window are done: `out` holds their normalised sums and `lse` max +
+        // log(sum) of their softmax, which is a running softmax with that max and a sum of 1
+        if (blocks_seen(last_pos, window, pool) == 0) return;       // no row of the tile sees a block
+        if (qrow < len) {
+            m_i = lse[(size_t)(start + qrow) * nh + h];
+            l_i = 1.f;
+            const size_t ob = (size_t)(start + qrow) * nh * dv + (size_t)h * dv;
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const int d = g + 8 * k;
+                if (d < dv) acc[k] = ld_f(out, dt, ob + d);
+            }
+        }
+    }
 
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < (lse ? 1 : 2); ++pass) {
         const void* kc = pass == 0 ? kpool : kcache;
         const void* vc = pass == 0 ? vpool : vcache;
         int lo, hi;
@@ -268,10 +290,10 @@ extern "C" int illm_attn_pooled_rows(const void* q, int q_stride, void* out, int
                                      const void* vpool, const int32_t* page_table, int table_stride,
                                      int page_size, int n_seqs, int max_rows, int nh, int nkv, int dk,
                                      int dv, float scale, const float* head_scale, int window, int pool,
-                                     void* stream) {
+                                     const float* lse, void* stream) {
     if (n_seqs < 0 || max_rows < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 || dv <= 0 ||
         dv > 256 || page_size <= 0 || !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535 || window <= 0 ||
-        pool < 0 || (pool > 0 && (!kpool || !vpool)) || nh * dk > q_stride)
+        pool < 0 || (pool > 0 && (!kpool || !vpool)) || nh * dk > q_stride || (lse && pool <= 0))
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_rows == 0) return ILLM_OK;
     const size_t lds = ((size_t)(PQ + PK) * (dk + 1) + (size_t)PK * (dv + 1) + PQ * (PK + 1)) * sizeof(float);
@@ -282,7 +304,7 @@ extern "C" int illm_attn_pooled_rows(const void* q, int q_stride, void* out, int
     hipLaunchKernelGGL(attn_pooled_rows_kernel, dim3((max_rows + PQ - 1) / PQ, nh, n_seqs), dim3(256), lds,
                        (hipStream_t)stream, q, q_stride, out, dt, cu, seq_slot, seq_start, kcache, vcache,
                        kpool, vpool, page_table, table_stride, page_size, nh, nkv, dk, dv, scale, head_scale,
-                       window, pool);
+                       window, pool, lse);
     return illm_launch_status();
 }
 
@@ -298,7 +320,8 @@ attn_pooled_decode_kernel(const void* __restrict__ q, int q_stride, void* __rest
                           const int32_t* __restrict__ page_table, int table_stride, int page_size,
                           const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_len,
                           int nh, int nkv, int dk, int dv, float scale,
-                          const float* __restrict__ head_scale, int window, int pool) {
+                          const float* __restrict__ head_scale, int window, int pool,
+                          const float* __restrict__ lse) {
     __shared__ float wacc[4][256];
     __shared__ float wm[4], wl[4];
     const int h = blockIdx.x, b = blockIdx.y;
@@ -307,7 +330,9 @@ attn_pooled_decode_kernel(const void* __restrict__ q, int q_stride, void* __rest
     const int kvh = h / (nh / nkv);
     const int seen = pool > 0 ? blocks_seen(len - 1, window, pool) : 0;
     const int lo = max(0, len - window);
-    const int n_keys = seen + (len - lo);
+    // with `lse` the window's tokens are done (`out` and `lse` hold their softmax): the pooled rows alone
+    if (lse && seen == 0) return;
+    const int n_keys = lse ? seen : seen + (len - lo);
     const float sc = scale * (head_scale ? head_scale[h] : 1.f);
     float qv[4], acc[4];
 #pragma unroll
@@ -372,15 +397,22 @@ attn_pooled_decode_kernel(const void* __restrict__ q, int q_stride, void* __rest
     __syncthreads();
     float mm = wm[0];
     for (int i = 1; i < 4; ++i) mm = fmaxf(mm, wm[i]);
+    const float m0 = lse ? lse[(size_t)b * nh + h] : NEG_INF;       // the window's softmax: max m0, sum 1
+    mm = fmaxf(mm, m0);
     float f[4], lt = 0.f;
     for (int i = 0; i < 4; ++i) {
         f[i] = wm[i] == NEG_INF ? 0.f : expf(wm[i] - mm);
         lt += f[i] * wl[i];
     }
+    const float f0 = lse ? expf(m0 - mm) : 0.f;
+    lt += f0;
     const float inv = 1.0f / lt;
-    for (int d = threadIdx.x; d < dv; d += 256)
-        st_f(out, dt, ((size_t)b * nh + h) * dv + d,
-             (f[0] * wacc[0][d] + f[1] * wacc[1][d] + f[2] * wacc[2][d] + f[3] * wacc[3][d]) * inv);
+    for (int d = threadIdx.x; d < dv; d += 256) {
+        const size_t at = ((size_t)b * nh + h) * dv + d;
+        float a = f[0] * wacc[0][d] + f[1] * wacc[1][d] + f[2] * wacc[2][d] + f[3] * wacc[3][d];
+        if (lse) a += f0 * ld_f(out, dt, at);
+        st_f(out, dt, at, a * inv);
+    }
 }
 
 extern "C" int illm_attn_pooled_decode(const void* q, int q_stride, void* out, int dt,
@@ -388,14 +420,15 @@ extern "C" int illm_attn_pooled_decode(const void* q, int q_stride, void* out, i
                                        const void* vpool, const int32_t* page_table, int table_stride,
                                        int page_size, const int32_t* seq_slot, const int32_t* seq_len,
                                        int B, int nh, int nkv, int dk, int dv, float scale,
-                                       const float* head_scale, int window, int pool, void* stream) {
+                                       const float* head_scale, int window, int pool, const float* lse,
+                                       void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dk > 256 || dv <= 0 || dv > 256 ||
         page_size <= 0 || !illm_dtype_ok(dt) || B > 65535 || window <= 0 || pool < 0 ||
-        (pool > 0 && (!kpool || !vpool)) || nh * dk > q_stride)
+        (pool > 0 && (!kpool || !vpool)) || nh * dk > q_stride || (lse && pool <= 0))
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     hipLaunchKernelGGL(attn_pooled_decode_kernel, dim3(nh, B), dim3(256), 0, (hipStream_t)stream, q,
                        q_stride, out, dt, kcache, vcache, kpool, vpool, page_table, table_stride, page_size,
-                       seq_slot, seq_len, nh, nkv, dk, dv, scale, head_scale, window, pool);
+                       seq_slot, seq_len, nh, nkv, dk, dv, scale, head_scale, window, pool, lse);
     return illm_launch_status();
 }

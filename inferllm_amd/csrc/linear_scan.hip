@@ -312,6 +312,7 @@ lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, cons
         float ar[LRU_ROWS], ai[LRU_ROWS];
 #pragma unroll
         for (int r = 0; r < LRU_ROWS; ++r) ar[r] = ai[r] = 0.f;
+#pragma unroll 8
         for (int i = 0; i < cb; ++i) {
             const float w1 = wr[(size_t)i * cb + o], w2 = wi[(size_t)i * cb + o];
 #pragma unroll
@@ -378,14 +379,102 @@ lru_scan_kernel(const float* __restrict__ a, const float* __restrict__ x, float*
     state[(size_t)slot * C + c] = S;
 }
 
+// The same recurrence for long steps, in three launches over chunks of LRU_CHUNK rows:
+//   lru_chunk_sums   per (sequence, chunk, channel): the chunk's product of decays P and its sum B
+//                    from a state of zero (S_end = P S_start + B)
+//   lru_chunk_carry  per (sequence, channel): the state at every chunk's start, chunk after chunk
+//                    (and the sequence's last state back into the slot)
+//   lru_chunk_apply  per (sequence, chunk, channel): the recurrence again from the chunk's start
+//                    state, with the other branch multiplied in
+// A row's state is then summed in another order than token by token: it differs in rounding only.
+#define LRU_CHUNK 32
+__global__ void __launch_bounds__(256)
+lru_chunk_sums_kernel(const float* __restrict__ a, const float* __restrict__ x, float* __restrict__ P,
+                      float* __restrict__ B, const int32_t* __restrict__ cu, int C, int max_chunks) {
+    const int b = blockIdx.z, ch = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    const int t0 = ch * LRU_CHUNK;
+    if (t0 >= n) return;
+    const int t1 = min(n, t0 + LRU_CHUNK);
+    float p = 1.f, s = 0.f;
+    for (int t = t0; t < t1; ++t) {
+        const size_t at = (size_t)(r0 + t) * C + c;
+        const float av = a[at];
+        s = fmaf(av, s, x[at]);
+        p *= av;
+    }
+    const size_t o = ((size_t)b * max_chunks + ch) * C + c;
+    P[o] = p;
+    B[o] = s;
+}
+
+__global__ void __launch_bounds__(256)
+lru_chunk_carry_kernel(const float* __restrict__ P, float* __restrict__ B, float* __restrict__ state,
+                       const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot, int C,
+                       int max_chunks) {
+    const int b = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int n = cu[b + 1] - cu[b];
+    if (n <= 0) return;
+    const int chunks = (n + LRU_CHUNK - 1) / LRU_CHUNK, slot = seq_slot[b];
+    float S = state[(size_t)slot * C + c];
+    for (int ch = 0; ch < chunks; ++ch) {
+        const size_t o = ((size_t)b * max_chunks + ch) * C + c;
+        const float next = fmaf(P[o], S, B[o]);
+        B[o] = S;                                   // the chunk's start state, for lru_chunk_apply
+        S = next;
+    }
+    state[(size_t)slot * C + c] = S;
+}
+
+__global__ void __launch_bounds__(256)
+lru_chunk_apply_kernel(const float* __restrict__ a, const float* __restrict__ x,
+                       const float* __restrict__ S0, const void* __restrict__ Y, int y_dt, int y_stride,
+                       int y_off, const float* __restrict__ yb, void* __restrict__ out, int out_dt,
+                       const int32_t* __restrict__ cu, int C, int max_chunks) {
+    const int b = blockIdx.z, ch = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    const int t0 = ch * LRU_CHUNK;
+    if (t0 >= n) return;
+    const int t1 = min(n, t0 + LRU_CHUNK);
+    float S = S0[((size_t)b * max_chunks + ch) * C + c];
+    const float bias = yb ? yb[c] : 0.f;
+    for (int t = t0; t < t1; ++t) {
+        const size_t at = (size_t)(r0 + t) * C + c;
+        S = fmaf(a[at], S, x[at]);
+        const float y = ls_gelu_tanh(ld_f(Y, y_dt, (size_t)(r0 + t) * y_stride + y_off + c) + bias);
+        st_f(out, out_dt, at, S * y);
+    }
+}
+
+// `scratch`: 2 * n_seqs * ceil(max_rows / 32) * C floats for steps of 64 rows a sequence or more
+// (null, or fewer rows: a thread walks its channel through the whole sequence).
 extern "C" int illm_lru_scan(const float* a, const float* x, float* state, const void* Y, int y_dt,
                              int y_stride, int y_off, const float* yb, void* out, int out_dt,
-                             const int32_t* cu, const int32_t* seq_slot, int n_seqs, int C, void* stream) {
+                             const int32_t* cu, const int32_t* seq_slot, int n_seqs, int max_rows, int C,
+                             float* scratch, void* stream) {
     if (n_seqs < 0 || C <= 0 || !illm_dtype_ok(y_dt) || !illm_dtype_ok(out_dt) || y_off < 0 ||
-        y_off + C > y_stride || n_seqs > 65535 * 32)
+        y_off + C > y_stride || n_seqs > 65535 || max_rows < 0)
         return ILLM_ERR_ARG;
     if (n_seqs == 0) return ILLM_OK;
-    hipLaunchKernelGGL(lru_scan_kernel, dim3(n_seqs, (C + 255) / 256), dim3(256), 0, (hipStream_t)stream, a,
-                       x, state, Y, y_dt, y_stride, y_off, yb, out, out_dt, cu, seq_slot, C);
+    hipStream_t st = (hipStream_t)stream;
+    const int cblocks = (C + 255) / 256;
+    if (scratch && max_rows >= 2 * LRU_CHUNK) {
+        const int chunks = (max_rows + LRU_CHUNK - 1) / LRU_CHUNK;
+        if (chunks > 65535) return ILLM_ERR_ARG;
+        float* P = scratch;
+        float* B = scratch + (size_t)n_seqs * chunks * C;
+        hipLaunchKernelGGL(lru_chunk_sums_kernel, dim3(cblocks, chunks, n_seqs), dim3(256), 0, st, a, x, P, B, cu,
+                           C, chunks);
+        hipLaunchKernelGGL(lru_chunk_carry_kernel, dim3(cblocks, n_seqs), dim3(256), 0, st, P, B, state, cu,
+                           seq_slot, C, chunks);
+        hipLaunchKernelGGL(lru_chunk_apply_kernel, dim3(cblocks, chunks, n_seqs), dim3(256), 0, st, a, x, B, Y,
+                           y_dt, y_stride, y_off, yb, out, out_dt, cu, C, chunks);
+        return illm_launch_status();
+    }
+    hipLaunchKernelGGL(lru_scan_kernel, dim3(n_seqs, cblocks), dim3(256), 0, st, a, x, state, Y, y_dt,
+                       y_stride, y_off, yb, out, out_dt, cu, seq_slot, C);
     return illm_launch_status();
 }

@@ -172,7 +172,30 @@ extern "C" int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, in
 //     out = h + sum_j conv_w[:, j] h(t - (taps - 1 - j))                (conv_w null: out = h)
 // With `row_idx` only those rows are formed and x is left as it is.  The convolution is for steps of
 // one row a sequence: the earlier inputs come from tail [slots][taps - 1][E], which is moved on.
-// grid (rows); 256 threads; the row's sum is kept in LDS (E floats) between the passes.
+// grid (rows); 256 threads.  A thread owns NV groups of 4 consecutive columns (E % 4 == 0, E <= 1024
+// NV) and asks for everything it reads of a pass before it uses any of it; other widths take the
+// plain loop (NV 0), which keeps the row's sum in LDS (E floats) between the passes.
+__device__ __forceinline__ float4 sc_ld4(const void* p, int dt, size_t i4) {
+    if (dt == ILLM_BF16) {
+        const uint2 u = ((const uint2*)p)[i4];
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+    }
+    return ((const float4*)p)[i4];
+}
+
+__device__ __forceinline__ void sc_st4(void* p, int dt, size_t i4, float4 v) {
+    if (dt == ILLM_BF16) {
+        uint2 u;
+        u.x = pack_bf16x2(v.x, v.y);
+        u.y = pack_bf16x2(v.z, v.w);
+        ((uint2*)p)[i4] = u;
+    } else {
+        ((float4*)p)[i4] = v;
+    }
+}
+
+template <int NV>
 __global__ void __launch_bounds__(256)
 post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a_dt,
                         const void* __restrict__ post_w, int post_w_dt, float post_eps, float gain,
@@ -185,6 +208,74 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
     const int r = blockIdx.x;
     const int in_row = row_idx ? row_idx[r] : r;
     const size_t ib = (size_t)in_row * E, ob = (size_t)r * E;
+    const int K = taps - 1;
+    const int slot = conv_w ? row_slot[r] : 0;
+    if (NV > 0) {
+        const int n4 = E / 4;
+        float4 xv[NV > 0 ? NV : 1], av[NV > 0 ? NV : 1];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int i4 = threadIdx.x + 256 * k;
+            xv[k] = i4 < n4 ? ((const float4*)(x + ib))[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            av[k] = (a && i4 < n4) ? sc_ld4(a, a_dt, ib / 4 + i4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        if (a) {
+            float sa = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) sa += av[k].x * av[k].x + av[k].y * av[k].y + av[k].z * av[k].z + av[k].w * av[k].w;
+            sa = block_sum(sa, red);
+            const float inv_a = 1.0f / sqrtf(sa / (float)E + post_eps);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int i4 = threadIdx.x + 256 * k;
+                if (i4 >= n4) continue;
+                const float4 pw = sc_ld4(post_w, post_w_dt, i4);
+                xv[k].x += gain * (av[k].x * inv_a * pw.x);
+                xv[k].y += gain * (av[k].y * inv_a * pw.y);
+                xv[k].z += gain * (av[k].z * inv_a * pw.z);
+                xv[k].w += gain * (av[k].w * inv_a * pw.w);
+                if (!row_idx) ((float4*)(x + ib))[i4] = xv[k];
+            }
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) ss += xv[k].x * xv[k].x + xv[k].y * xv[k].y + xv[k].z * xv[k].z + xv[k].w * xv[k].w;
+        ss = block_sum(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int i4 = threadIdx.x + 256 * k;
+            if (i4 >= n4) continue;
+            const float4 wv = sc_ld4(w, w_dt, i4);
+            float h[4] = {(xv[k].x * scale) * wv.x, (xv[k].y * scale) * wv.y, (xv[k].z * scale) * wv.z,
+                          (xv[k].w * scale) * wv.w};
+            if (conv_w) {
+                float4 old[CONV_MAX_TAPS - 1];
+#pragma unroll
+                for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
+                    if (j < K) old[j] = sc_ld4(tail, tail_dt, ((size_t)slot * K + j) * n4 + i4);
+                float hq[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    hq[e] = conv_round(h[e], out_dt);
+                    const float* cw = conv_w + (size_t)(4 * i4 + e) * taps;
+                    float c = 0.f;
+#pragma unroll
+                    for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
+                        if (j < K) c = fmaf(cw[j], ((const float*)&old[j])[e], c);
+                    c = fmaf(cw[K], hq[e], c);
+                    h[e] = hq[e] + c;
+                }
+                // the tail moves on by the new input
+#pragma unroll
+                for (int j = 1; j < CONV_MAX_TAPS - 1; ++j)
+                    if (j < K) sc_st4(tail, tail_dt, ((size_t)slot * K + (j - 1)) * n4 + i4, old[j]);
+                sc_st4(tail, tail_dt, ((size_t)slot * K + (K - 1)) * n4 + i4, make_float4(hq[0], hq[1], hq[2], hq[3]));
+            }
+            sc_st4(out, out_dt, ob / 4 + i4, make_float4(h[0], h[1], h[2], h[3]));
+        }
+        return;
+    }
     float inv_a = 0.f;
     if (a) {
         float sa = 0.f;
@@ -207,13 +298,10 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
     }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)E + eps);
-    const int K = taps - 1;
-    const int slot = conv_w ? row_slot[r] : 0;
     for (int i = threadIdx.x; i < E; i += 256) {
         float h = (row[i] * scale) * ld_f(w, w_dt, i);
         if (conv_w) {
             h = conv_round(h, out_dt);
-            float y = h;
             float in[CONV_MAX_TAPS];
 #pragma unroll
             for (int j = 0; j < CONV_MAX_TAPS; ++j) {
@@ -224,11 +312,10 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
 #pragma unroll
             for (int j = 0; j < CONV_MAX_TAPS; ++j)
                 if (j < taps) c = fmaf(conv_w[(size_t)i * taps + j], in[j], c);
-            y += c;
 #pragma unroll
             for (int j = 1; j < CONV_MAX_TAPS; ++j)
                 if (j < taps) st_f(tail, tail_dt, ((size_t)slot * K + (j - 1)) * E + i, in[j]);
-            h = y;
+            h += c;
         }
         st_f(out, out_dt, ob + i, h);
     }
@@ -244,14 +331,25 @@ extern "C" int illm_post_add_rmsnorm(float* x, const void* a, int a_dt, const vo
         (conv_w && (taps < 2 || taps > CONV_MAX_TAPS || !tail || !row_slot || row_idx || !illm_dtype_ok(tail_dt))))
         return ILLM_ERR_ARG;
     if (rows == 0) return ILLM_OK;
+    hipStream_t st = (hipStream_t)stream;
+#define GO(NV_, LDS_)                                                                                   \
+    hipLaunchKernelGGL(post_add_rmsnorm_kernel<NV_>, dim3(rows), dim3(256), LDS_, st, x, a, a_dt, post_w,   \
+                       post_w_dt, post_eps, gain, w, w_dt, out, out_dt, row_idx, E, eps, conv_w, taps, tail, \
+                       tail_dt, row_slot)
+    if (E % 4 == 0 && E <= 8192) {
+        if (E <= 1024) GO(1, 0);
+        else if (E <= 2048) GO(2, 0);
+        else if (E <= 4096) GO(4, 0);
+        else GO(8, 0);
+        return illm_launch_status();
+    }
     const size_t lds = (size_t)E * sizeof(float);
     if (lds > 64 * 1024) return ILLM_ERR_ARG;
     if (lds > 48 * 1024 &&
-        hipFuncSetAttribute((const void*)post_add_rmsnorm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute((const void*)post_add_rmsnorm_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess)
         return ILLM_ERR_LAUNCH;
-    hipLaunchKernelGGL(post_add_rmsnorm_kernel, dim3(rows), dim3(256), lds, (hipStream_t)stream, x, a, a_dt,
-                       post_w, post_w_dt, post_eps, gain, w, w_dt, out, out_dt, row_idx, E, eps, conv_w, taps,
-                       tail, tail_dt, row_slot);
+    GO(0, lds);
+#undef GO
     return illm_launch_status();
 }

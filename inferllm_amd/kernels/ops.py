@@ -1515,6 +1515,12 @@ def _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, what, gate_heads=False):
           f"{what}: gate rows of the queries' dtype with {nh * dv} columns from {gate_off}")
 
 
+def _lse_ok(lse, rows, nh, what):
+    if lse is not None:
+        _gpu(lse)
+        _need(lse.dtype == torch.float32 and lse.shape == (rows, nh), f"{what}: lse float32 [{rows}, {nh}]")
+
+
 def qkv_norm_mix_store(rows: torch.Tensor, k_off: int, v_off: int, q_weight: Optional[torch.Tensor],
                        k_weight: Optional[torch.Tensor], eps: float, lam: Optional[torch.Tensor],
                        first: Optional[torch.Tensor], first_off: int, row_pos: torch.Tensor,
@@ -1556,14 +1562,16 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
                   nh: int, nkv: int, dk: int, dv: int, scale: float, cap: float,
                   window: int, slopes: Optional[torch.Tensor] = None, chunk: int = 0,
                   gate: Optional[torch.Tensor] = None, gate_off: int = 0,
-                  gate_heads: bool = False) -> torch.Tensor:
+                  gate_heads: bool = False, lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of a step's packed rows over the paged cache (which holds the step's own
     keys and values by now): row r of sequence b stands at position seq_start[b] + r; scores
     cap tanh(q . k scale / cap) (cap 0: none); queries and keys of width dk, values of dv.
     `slopes` float32 [nh]: score -= slopes[h] (i - j).  `chunk` > 0: a row sees only the keys of its
     own chunk of positions.  `gate` [T, n] (columns gate_off ..): out *= sigmoid(gate), one
-    number a head and value dim, or with `gate_heads` one a head.  Returns [T, nh dv]."""
+    number a head and value dim, or with `gate_heads` one a head.  `lse` float32 [T, nh] takes
+    max + log(sum) of every row's and head's softmax.  Returns [T, nh dv]."""
     _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_rows", gate_heads)
+    _lse_ok(lse, q.shape[0], nh, "attn_cap_rows")
     _gpu(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
     _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_rows")
@@ -1572,7 +1580,7 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
         _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh, nkv,
         dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk), _p(gate),
-        gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _stream()),
+        gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _p(lse), _stream()),
         f"attn_cap_rows (sizes {dk}, {dv})")
     return out
 
@@ -1582,10 +1590,12 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                     seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
                     cap: float, window: int, nsplit: int, slopes: Optional[torch.Tensor] = None,
                     chunk: int = 0, gate: Optional[torch.Tensor] = None, gate_off: int = 0,
-                    gate_heads: bool = False) -> torch.Tensor:
+                    gate_heads: bool = False, lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for one new token per sequence: row b of q against the seq_len[b] keys
     (the new one included) of its slot, the keys cut into `nsplit` ranges.  Returns [B, nh dv]."""
     _cap_extras_ok(q, slopes, gate, gate_off, nh, dv, "attn_cap_decode", gate_heads)
+    _lse_ok(lse, q.shape[0], nh, "attn_cap_decode")
+    _need(lse is None or nsplit >= 2, "attn_cap_decode: lse comes from the merge of two or more ranges")
     _gpu(q, kcache, vcache, page_table, seq_slot, seq_len)
     B = q.shape[0]
     _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
@@ -1596,8 +1606,8 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(page_table),
         page_table.shape[1], page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh,
         nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _p(slopes), int(chunk),
-        _p(gate), gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _stream()),
-        f"attn_cap_decode (sizes {dk}, {dv})")
+        _p(gate), gate.shape[1] if gate is not None else 0, gate_off, 1 if gate_heads else 0, _p(lse),
+        _stream()), f"attn_cap_decode (sizes {dk}, {dv})")
     return out
 
 
@@ -1924,13 +1934,18 @@ def qk_rotate_store(rows: torch.Tensor, k_off: int, v_off: int, cos_sin: Optiona
                     rot: int, pairing: int, unit_norm: bool, eps: float, row_pos: torch.Tensor,
                     row_slot: torch.Tensor, kcache: Optional[torch.Tensor],
                     vcache: Optional[torch.Tensor], page_table: Optional[torch.Tensor], page_size: int,
-                    ring: int, nh: int, nkv: int, dk: int, dv: int) -> None:
+                    ring: int, nh: int, nkv: int, dk: int, dv: int,
+                    q_scale: Optional[torch.Tensor] = None) -> None:
     """In place on packed rows [q (nh dk) | .. k at k_off (nkv dk) | v at v_off (nkv dv)], in float32:
     the first `rot` dims of every q and k head turned by the row's position (cos_sin float32
     [positions, rot / 2, 2]; pairing 0: i with i + rot / 2, 1: 2i with 2i + 1), then with `unit_norm`
-    every head divided by its root mean square; k and v stored in the paged cache K [pages, nkv,
-    page_size, dk], V [pages, nkv, page_size, dv] (None: not stored; nkv 0: rows of queries alone)."""
-    _gpu(rows, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
+    every head divided by its root mean square, then query head h times `q_scale`[h] (float32 [nh]:
+    a scale of the scores that differs by head, taken into the queries); k and v stored in the paged
+    cache K [pages, nkv, page_size, dk], V [pages, nkv, page_size, dv] (None: not stored; nkv 0: rows
+    of queries alone)."""
+    _gpu(rows, cos_sin, row_pos, row_slot, kcache, vcache, page_table, q_scale)
+    _need(q_scale is None or (q_scale.dtype == torch.float32 and q_scale.shape == (nh,)),
+          f"qk_rotate_store: q_scale float32 [{nh}]")
     T = rows.shape[0]
     _i32(row_pos, T); _i32(row_slot, T); _i32(page_table)
     _need(rows.dim() == 2, "qk_rotate_store: rows [T, n]")
@@ -1944,7 +1959,7 @@ def qk_rotate_store(rows: torch.Tensor, k_off: int, v_off: int, cos_sin: Optiona
     _check(_lib().illm_qk_rotate_store(
         _p(rows), _code(rows), rows.shape[1], k_off, v_off, _p(cos_sin), rot if cos_sin is not None else 0,
         pairing, cos_sin.shape[0] if cos_sin is not None else 0, 1 if unit_norm else 0, ctypes.c_float(eps),
-        _p(row_pos), _p(row_slot), _p(kcache), _p(vcache), _p(page_table),
+        _p(q_scale), _p(row_pos), _p(row_slot), _p(kcache), _p(vcache), _p(page_table),
         page_table.shape[1] if page_table is not None else 0, page_size, ring, T, nh, nkv, dk, dv,
         _stream()), "qk_rotate_store")
 
@@ -1979,25 +1994,39 @@ def _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, 
               f"{what}: pooled rows laid out like the cache")
 
 
+def _pooled_out(q, nh, dv, pool, out, lse, what):
+    if lse is None:
+        _need(out is None, f"{what}: `out` is given together with `lse`")
+        return torch.empty((q.shape[0], nh * dv), dtype=q.dtype, device=q.device)
+    _gpu(out)
+    _lse_ok(lse, q.shape[0], nh, what)
+    _need(pool > 0 and out is not None and out.dtype == q.dtype and out.shape == (q.shape[0], nh * dv),
+          f"{what}: with `lse`, `out` [{q.shape[0]}, {nh * dv}] of the queries' dtype and pooled blocks")
+    return out
+
+
 def attn_pooled_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
                      seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                      kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
                      page_table: torch.Tensor, page_size: int, n_seqs: int, max_rows: int, nh: int,
                      nkv: int, dk: int, dv: int, scale: float, head_scale: Optional[torch.Tensor],
-                     window: int, pool: int) -> torch.Tensor:
+                     window: int, pool: int, out: Optional[torch.Tensor] = None,
+                     lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of a step's packed rows over the paged cache (which holds the step's own keys and
     values, and the pooled rows of the blocks it completed, by now): the row at position i sees
     tokens j with 0 <= i - j < window and pooled block b if b pool + pool - 1 <= i - window, in one
-    softmax; score = q . k scale head_scale[h].  Returns [T, nh dv]."""
+    softmax; score = q . k scale head_scale[h].  Returns [T, nh dv].  With `out` and `lse` (what
+    `attn_cap_rows` with that window left: the tokens' normalised sums and max + log(sum) of their
+    softmax) only the pooled blocks are gone through and merged into `out` in place."""
     _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, head_scale, pool,
                "attn_pooled_rows")
     _gpu(cu_seqlens, seq_slot, seq_start)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs)
-    out = torch.empty((q.shape[0], nh * dv), dtype=q.dtype, device=q.device)
+    out = _pooled_out(q, nh, dv, pool, out, lse, "attn_pooled_rows")
     _check(_lib().illm_attn_pooled_rows(
         _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(kpool), _p(vpool), _p(page_table), page_table.shape[1], page_size, n_seqs, max_rows,
-        nh, nkv, dk, dv, ctypes.c_float(scale), _p(head_scale), int(window), int(pool), _stream()),
+        nh, nkv, dk, dv, ctypes.c_float(scale), _p(head_scale), int(window), int(pool), _p(lse), _stream()),
         f"attn_pooled_rows (sizes {dk}, {dv})")
     return out
 
@@ -2006,18 +2035,20 @@ def attn_pooled_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tens
                        kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
                        page_table: torch.Tensor, page_size: int, seq_slot: torch.Tensor,
                        seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
-                       head_scale: Optional[torch.Tensor], window: int, pool: int) -> torch.Tensor:
-    """The same attention for one new token per sequence, at position seq_len[b] - 1.  Returns [B, nh dv]."""
+                       head_scale: Optional[torch.Tensor], window: int, pool: int,
+                       out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same attention for one new token per sequence, at position seq_len[b] - 1 (`out` and `lse`
+    as above, from `attn_cap_decode`).  Returns [B, nh dv]."""
     _pooled_ok(q, kcache, vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, head_scale, pool,
                "attn_pooled_decode")
     _gpu(seq_slot, seq_len)
     B = q.shape[0]
     _i32(seq_slot, B); _i32(seq_len, B)
-    out = torch.empty((B, nh * dv), dtype=q.dtype, device=q.device)
+    out = _pooled_out(q, nh, dv, pool, out, lse, "attn_pooled_decode")
     _check(_lib().illm_attn_pooled_decode(
         _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(kpool), _p(vpool), _p(page_table),
         page_table.shape[1], page_size, _p(seq_slot), _p(seq_len), B, nh, nkv, dk, dv, ctypes.c_float(scale),
-        _p(head_scale), int(window), int(pool), _stream()), f"attn_pooled_decode (sizes {dk}, {dv})")
+        _p(head_scale), int(window), int(pool), _p(lse), _stream()), f"attn_pooled_decode (sizes {dk}, {dv})")
     return out
 
 
@@ -2067,9 +2098,12 @@ def lru_gates(u: torch.Tensor, w_t: torch.Tensor, r_bias: torch.Tensor, i_bias: 
 
 def lru_scan(a: torch.Tensor, x: torch.Tensor, state: torch.Tensor, Y: torch.Tensor, y_off: int,
              y_bias: Optional[torch.Tensor], cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
-             n_seqs: int, out_dtype: torch.dtype) -> torch.Tensor:
+             n_seqs: int, max_rows: int, out_dtype: torch.dtype) -> torch.Tensor:
     """S <- a S + x per channel over every sequence's rows in order, from `state` float32 [slots, C]
-    and back into it; returns S gelu_tanh(Y[:, y_off ..] + y_bias) as [T, C]."""
+    and back into it; returns S gelu_tanh(Y[:, y_off ..] + y_bias) as [T, C].  `max_rows`: the most
+    rows a sequence brings; from 64 on the rows are gone through in chunks of 32 in parallel (a chunk's
+    product of decays and sum first, then the chunks' start states in order, then the rows), which
+    sums a row's state in another order than token by token."""
     _gpu(a, x, state, Y, y_bias, cu_seqlens, seq_slot)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
     T, C = a.shape
@@ -2078,9 +2112,12 @@ def lru_scan(a: torch.Tensor, x: torch.Tensor, state: torch.Tensor, Y: torch.Ten
           and Y.dim() == 2 and Y.shape[0] == T and y_off + C <= Y.shape[1], "lru_scan: shapes")
     _need(y_bias is None or (y_bias.dtype == torch.float32 and y_bias.shape == (C,)), "lru_scan: y_bias float32 [C]")
     out = torch.empty((T, C), dtype=out_dtype, device=a.device)
+    scratch = None
+    if max_rows >= 64:
+        scratch = torch.empty((2, n_seqs, -(-max_rows // 32), C), dtype=torch.float32, device=a.device)
     _check(_lib().illm_lru_scan(_p(a), _p(x), _p(state), _p(Y), _code(Y), Y.shape[1], y_off, _p(y_bias),
-                                _p(out), _code(out), _p(cu_seqlens), _p(seq_slot), n_seqs, C, _stream()),
-           "lru_scan")
+                                _p(out), _code(out), _p(cu_seqlens), _p(seq_slot), n_seqs, int(max_rows), C,
+                                _p(scratch), _stream()), "lru_scan")
     return out
 
 

@@ -248,7 +248,8 @@ class GatedAttention(Mixer):
       "interleaved"; the cache keeps the turned keys;
     * `qk_norm` "head": after the rotation every q and k head is divided by its own root mean
       square (`eps`), without a weight;
-    * `head_scale`: the score of head h is multiplied by the stored `head_scale`[h];
+    * `head_scale`: the score of head h is multiplied by the stored `head_scale`[h] (taken into the
+      queries, in float32, behind the rotation and the norm a head);
     * `pool` P > 0 (with `window`): beside the last `window` tokens a row sees one pooled key and
       value for every block of P tokens that lies wholly before its window (block b if
       b P + P - 1 <= i - window): the means of the block's keys and values as the cache holds them,
@@ -275,10 +276,12 @@ class GatedAttention(Mixer):
             raise ValueError(f"gated attention: qk_norm {qk_norm!r} or gate {gate!r}: False, True or 'head'")
         if int(pool or 0) and not window:
             raise ValueError("gated attention: pooled blocks lie before a window; `pool` needs `window`")
-        if (int(pool or 0) or head_scale) and (gate or chunk or softcap or slope_power or value_mix
-                                               or qk_norm is True):
-            raise ValueError("gated attention: pooled blocks and a scale a head go with a window, a rotation "
-                             "and the norm a head, not with a gate, chunks, a cap, slopes or mixed values")
+        if int(pool or 0) and (gate or chunk or softcap or slope_power):
+            raise ValueError("gated attention: pooled blocks go with a window alone, not with a gate, "
+                             "chunks, a cap or slopes")
+        if head_scale and (softcap or qk_norm is True or value_mix):
+            raise ValueError("gated attention: a scale a head is taken into the queries behind the rotation "
+                             "and the norm a head; it goes with neither a cap, a norm over all heads nor mixed values")
         if not own_kv and (value_mix or qk_norm is True):
             raise ValueError("gated attention: a layer that reads another layer's keys mixes and norms none")
         if num_heads % num_kv_heads:
@@ -364,7 +367,7 @@ class GatedAttention(Mixer):
                                 0 if position is None or position.pairing == "half" else 1,
                                 self.qk_norm == "head", self.eps, ctx.row_pos, ctx.row_slot,
                                 kc if store else None, vc if store else None, group.table, group.page_size,
-                                group.ring, nh, nkv if self.own_kv else 0, dk, dv)
+                                group.ring, nh, nkv if self.own_kv else 0, dk, dv, q_scale=self.head_scale)
         else:
             first, first_off = None, 0
             if self.value_mix == "mixed":
@@ -377,31 +380,29 @@ class GatedAttention(Mixer):
                                    group.page_size, group.ring, nh, nkv, dk, dv)
             if self.value_mix == "source":
                 ctx.exchange["value_mix_source"] = (rows, self.v_off, nkv * dv)
-        if self.pool or self.has_head_scale:
-            kp = vp = None
-            if self.pool:
-                line_tensors, _ = ctx.cache.token_line(line)
-                kp, vp = line_tensors["kp"], line_tensors["vp"]
-                if store:
-                    ops.pool_store(ctx.row_pos, ctx.row_slot, kc, vc, kp, vp, group.table, group.page_size,
-                                   nkv, dk, dv, self.pool)
-            seen = window or (1 << 30)
-            if ctx.prefill:
-                o = ops.attn_pooled_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, kp, vp,
-                                         group.table, group.page_size, ctx.n_seqs, ctx.max_rows, nh, nkv, dk,
-                                         dv, self.scale, self.head_scale, seen, self.pool)
-            else:
-                o = ops.attn_pooled_decode(rows, kc, vc, kp, vp, group.table, group.page_size, ctx.seq_slot,
-                                           ctx.seq_len, nh, nkv, dk, dv, self.scale, self.head_scale, seen,
-                                           self.pool)
-            return ops.linear(o, self.w_o)
         gate = rows if self.gate else None
         by_head = self.gate == "head"
+        # pooled blocks before the window: the window's tokens by the kernels below, which leave max +
+        # log(sum) of each softmax; then the blocks are merged in.  A step none of whose rows can see
+        # a block (`ctx.max_len` bounds the positions) has the window alone.
+        kp = vp = lse = None
+        if self.pool:
+            line_tensors, _ = ctx.cache.token_line(line)
+            kp, vp = line_tensors["kp"], line_tensors["vp"]
+            if store:
+                ops.pool_store(ctx.row_pos, ctx.row_slot, kc, vc, kp, vp, group.table, group.page_size,
+                               nkv, dk, dv, self.pool)
+            if ctx.max_len - window >= self.pool:
+                lse = torch.empty((rows.shape[0], nh), dtype=torch.float32, device=rows.device)
         if ctx.prefill:
             o = ops.attn_cap_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, group.table,
                                   group.page_size, group.ring, ctx.n_seqs, ctx.max_rows, nh, nkv, dk, dv,
                                   self.scale, self.softcap, window, self.slopes, self.chunk, gate, self.g_off,
-                                  by_head)
+                                  by_head, lse)
+            if lse is not None:
+                ops.attn_pooled_rows(rows, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, kp, vp,
+                                     group.table, group.page_size, ctx.n_seqs, ctx.max_rows, nh, nkv, dk, dv,
+                                     self.scale, None, window, self.pool, out=o, lse=lse)
         else:
             longest = ctx.max_len
             for bound in (window, self.chunk):
@@ -411,7 +412,13 @@ class GatedAttention(Mixer):
             # (measured: more ranges than that cost more in set-up and merging than they hide)
             blocks = ctx.n_seqs * nkv * -(-(nh // nkv) // 4)
             nsplit = max(1, min(-(-512 // max(1, blocks)), 16, tiles))
+            if lse is not None:
+                nsplit = max(nsplit, 2)              # the kernel that merges the ranges writes `lse`
             o = ops.attn_cap_decode(rows, kc, vc, group.table, group.page_size, group.ring, ctx.seq_slot,
                                     ctx.seq_len, nh, nkv, dk, dv, self.scale, self.softcap, window,
-                                    nsplit, self.slopes, self.chunk, gate, self.g_off, by_head)
+                                    nsplit, self.slopes, self.chunk, gate, self.g_off, by_head, lse)
+            if lse is not None:
+                ops.attn_pooled_decode(rows, kc, vc, kp, vp, group.table, group.page_size, ctx.seq_slot,
+                                       ctx.seq_len, nh, nkv, dk, dv, self.scale, None, window, self.pool,
+                                       out=o, lse=lse)
         return ops.linear(o, self.w_o)

@@ -309,5 +309,6 @@ class GatedLinearRecurrence(Mixer):
             ops.short_conv_tail(U, C, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps,
                                 in_bias=self.x_bias)
         a, x = ops.lru_gates(u, self.w_gates, self.r_bias, self.i_bias, self.lam, LRU_RATE)
-        y = ops.lru_scan(a, x, S, U, 0, self.y_bias, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, ctx.act_dtype)
+        y = ops.lru_scan(a, x, S, U, 0, self.y_bias, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs,
+                         ctx.max_rows if ctx.prefill else 1, ctx.act_dtype)
         return ops.linear(y, self.w_o)

@@ -443,8 +443,9 @@ def kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table,
         vcache[page, :, at, :] = rows[r, v_off:v_off + nkv * dv].view(nkv, dv)
 
 
-def _attend_capped(q, k, v, scale, cap, slopes=None):
-    """q [nh, dk], k [L, nkv, dk], v [L, nkv, dv]: every key visible, the last one the query's own."""
+def _attend_capped(q, k, v, scale, cap, slopes=None, lse=None):
+    """q [nh, dk], k [L, nkv, dk], v [L, nkv, dv]: every key visible, the last one the query's own.
+    `lse` [nh] takes log(sum(exp(score))) of every head."""
     nh, per, L = q.shape[0], q.shape[0] // k.shape[1], k.shape[0]
     out = torch.zeros(nh, v.shape[2], dtype=F64)
     for h in range(nh):
@@ -454,6 +455,8 @@ def _attend_capped(q, k, v, scale, cap, slopes=None):
         if slopes is not None:
             s = s - slopes[h].to(F64) * torch.arange(L - 1, -1, -1, dtype=F64)
         out[h] = torch.softmax(s, dim=0) @ v[:, h // per, :].to(F64)
+        if lse is not None:
+            lse[h] = torch.logsumexp(s, dim=0).to(lse.dtype)
     return out
 
 
@@ -494,7 +497,7 @@ def _cached(kcache, vcache, page_table, slot, first, total, page_size, ring):
 
 def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, page_size, ring,
                   n_seqs, max_rows, nh, nkv, dk, dv, scale, cap, window, slopes=None, chunk=0, gate=None,
-                  gate_off=0, gate_heads=False):
+                  gate_off=0, gate_heads=False, lse=None):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(n_seqs):
         s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
@@ -502,19 +505,22 @@ def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table
             pos = int(seq_start[b]) + a
             first = _first_seen(pos, window, chunk)
             k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, pos + 1, page_size, ring)
-            row = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
+            row = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap, slopes,
+                                 lse[s0 + a] if lse is not None else None).reshape(-1)
             out[s0 + a] = _gated(row, gate, s0 + a, gate_off, nh if gate_heads else 0).to(q.dtype)
     return out
 
 
 def attn_cap_decode(q, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, dk, dv,
-                    scale, cap, window, nsplit, slopes=None, chunk=0, gate=None, gate_off=0, gate_heads=False):
+                    scale, cap, window, nsplit, slopes=None, chunk=0, gate=None, gate_off=0, gate_heads=False,
+                    lse=None):
     out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
     for b in range(q.shape[0]):
         n = int(seq_len[b])
         first = _first_seen(n - 1, window, chunk)
         k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, n, page_size, ring)
-        row = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap, slopes).reshape(-1)
+        row = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap, slopes,
+                             lse[b] if lse is not None else None).reshape(-1)
         out[b] = _gated(row, gate, b, gate_off, nh if gate_heads else 0).to(q.dtype)
     return out
 
@@ -758,7 +764,7 @@ def clamped_swish_mul(gate_up, limit):
 
 # ---------------------------------------------------------------- attention over a window and pooled blocks
 def qk_rotate_store(rows, k_off, v_off, cos_sin, rot, pairing, unit_norm, eps, row_pos, row_slot, kcache,
-                    vcache, page_table, page_size, ring, nh, nkv, dk, dv):
+                    vcache, page_table, page_size, ring, nh, nkv, dk, dv, q_scale=None):
     half = rot // 2
     for r in range(rows.shape[0]):
         for off, heads in ((0, nh), (k_off, nkv)):
@@ -773,6 +779,8 @@ def qk_rotate_store(rows, k_off, v_off, cos_sin, rot, pairing, unit_norm, eps, r
                 x[:, ia], x[:, ib] = u * c - v * s, v * c + u * s
             if unit_norm:
                 x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+            if q_scale is not None and off == 0:
+                x = x * q_scale.to(F64)[:, None]
             rows[r, off:off + heads * dk] = x.reshape(-1).to(rows.dtype)
     if kcache is not None:
         kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table, page_size, ring, nkv, dk, dv)
@@ -807,8 +815,10 @@ def _attend_pooled(q, pos, slot, kcache, vcache, kpool, vpool, page_table, page_
 
 
 def attn_pooled_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, kpool, vpool, page_table, page_size,
-                     n_seqs, max_rows, nh, nkv, dk, dv, scale, head_scale, window, pool):
-    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+                     n_seqs, max_rows, nh, nkv, dk, dv, scale, head_scale, window, pool, out=None, lse=None):
+    # (with `out` and `lse`, what the window's kernel left, the kernel merges the pooled blocks in;
+    # the result is the whole attention either way)
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype) if out is None else out
     for b in range(n_seqs):
         s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
         for a in range(s1 - s0):
@@ -819,8 +829,8 @@ def attn_pooled_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, kpool, 
 
 
 def attn_pooled_decode(q, kcache, vcache, kpool, vpool, page_table, page_size, seq_slot, seq_len, nh, nkv, dk,
-                       dv, scale, head_scale, window, pool):
-    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+                       dv, scale, head_scale, window, pool, out=None, lse=None):
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype) if out is None else out
     for b in range(q.shape[0]):
         out[b] = _attend_pooled(q[b, :nh * dk].view(nh, dk), int(seq_len[b]) - 1, int(seq_slot[b]), kcache,
                                 vcache, kpool, vpool, page_table, page_size, nh, nkv, dk, dv, scale, head_scale,
@@ -852,7 +862,7 @@ def lru_gates(u, w_t, r_bias, i_bias, lam, rate):
     return a.to(torch.float32), x.to(torch.float32)
 
 
-def lru_scan(a, x, state, Y, y_off, y_bias, cu_seqlens, seq_slot, n_seqs, out_dtype):
+def lru_scan(a, x, state, Y, y_off, y_bias, cu_seqlens, seq_slot, n_seqs, max_rows, out_dtype):
     T, C = a.shape
     out = torch.zeros(T, C, dtype=F64)
     y = Y[:, y_off:y_off + C].to(F64) + (y_bias.to(F64) if y_bias is not None else 0.0)

@@ -512,11 +512,13 @@ def test_pooled_window_attention_against_plain_torch(dtype):
         vc = torch.randn(pages, nkv, page, dv, generator=g).to(dtype)
         kp, vp = torch.randn(kc.shape, generator=g).to(dtype), torch.randn(vc.shape, generator=g).to(dtype)
         r_want, kc_want, vc_want = rows.clone(), kc.clone(), vc.clone()
+        qs = torch.rand(nh, generator=g) + 0.5 if pairing else None        # a scale a query head, or none
         R.qk_rotate_store(r_want, k_off, v_off, cs, rot, pairing, True, 1e-5, row_pos, row_slot, kc_want, vc_want,
-                          table, page, 0, nh, nkv, dk, dv)
+                          table, page, 0, nh, nkv, dk, dv, qs)
         r_got, kc_got, vc_got = rows.cuda(), kc.cuda(), vc.cuda()
         ops.qk_rotate_store(r_got, k_off, v_off, cs.cuda() if rot else None, rot, pairing, True, 1e-5, row_pos.cuda(),
-                            row_slot.cuda(), kc_got, vc_got, table.cuda(), page, 0, nh, nkv, dk, dv)
+                            row_slot.cuda(), kc_got, vc_got, table.cuda(), page, 0, nh, nkv, dk, dv,
+                            qs.cuda() if qs is not None else None)
         _near(r_got, r_want, tol); _near(kc_got, kc_want, tol); _near(vc_got, vc_want, tol)
         kp_want, vp_want, kp_got, vp_got = kp.clone(), vp.clone(), kp.cuda(), vp.cuda()
         if pool:
@@ -545,6 +547,22 @@ def test_pooled_window_attention_against_plain_torch(dtype):
             got = ops.attn_pooled_decode(q1.cuda(), *ins[1:], table.cuda(), page, seq_slot.cuda(), seq_len.cuda(),
                                          nh, nkv, dk, dv, 0.3, hs.cuda() if hs is not None else None, window, pool)
             _near(got, want[last], tol)
+            if pool and hs is None:
+                # the window's tokens by the capped attention's kernels, which leave max + log(sum) of
+                # every softmax, then the pooled blocks merged in: the same attention
+                lse = torch.empty(T, nh, dtype=torch.float32, device="cuda")
+                o = ops.attn_cap_rows(ins[0], cu.cuda(), seq_slot.cuda(), seq_start.cuda(), ins[1], ins[2],
+                                      table.cuda(), page, 0, 3, max(lens), nh, nkv, dk, dv, 0.3, 0.0, window,
+                                      lse=lse)
+                ops.attn_pooled_rows(ins[0], cu.cuda(), seq_slot.cuda(), seq_start.cuda(), *ins[1:], table.cuda(),
+                                     page, 3, max(lens), nh, nkv, dk, dv, 0.3, None, window, pool, out=o, lse=lse)
+                _near(o, want, 2 * tol)
+                lse1 = torch.empty(3, nh, dtype=torch.float32, device="cuda")
+                o1 = ops.attn_cap_decode(q1.cuda(), ins[1], ins[2], table.cuda(), page, 0, seq_slot.cuda(),
+                                         seq_len.cuda(), nh, nkv, dk, dv, 0.3, 0.0, window, 2, lse=lse1)
+                ops.attn_pooled_decode(q1.cuda(), *ins[1:], table.cuda(), page, seq_slot.cuda(), seq_len.cuda(), nh,
+                                       nkv, dk, dv, 0.3, None, window, pool, out=o1, lse=lse1)
+                _near(o1, want[last], 2 * tol)
 
 
 @pytest.mark.parametrize("matrix_cores", [1, 0])
@@ -591,7 +609,7 @@ def test_linear_attention_and_recurrent_unit_kernels_against_plain_torch(dtype):
     of 8 to 300 channels, a state that goes on from what the slot holds."""
     from inferllm_amd.kernels import ops
     g = torch.Generator().manual_seed(11)
-    for lens in ([70, 1, 19], [1, 1, 1]):
+    for lens in ([70, 1, 19], [1, 1, 1], [200, 64, 33]):      # from 64 rows on the scan runs in chunks
         T = sum(lens)
         cu, seq_slot, _ = _packed(lens, [2, 0, 4])
         for H, dk, dv in ((3, 10, 14), (1, 40, 9)):
@@ -614,6 +632,7 @@ def test_linear_attention_and_recurrent_unit_kernels_against_plain_torch(dtype):
             yb = torch.randn(C, generator=g)
             state = torch.randn(6, C, generator=g)
             s_want, s_got = state.clone(), state.cuda()
-            want = R.lru_scan(a_want, x_want, s_want, Y, 5, yb, cu, seq_slot, 3, torch.float32)
-            got = ops.lru_scan(a_got, x_got, s_got, Y.cuda(), 5, yb.cuda(), cu.cuda(), seq_slot.cuda(), 3, torch.float32)
+            want = R.lru_scan(a_want, x_want, s_want, Y, 5, yb, cu, seq_slot, 3, max(lens), torch.float32)
+            got = ops.lru_scan(a_got, x_got, s_got, Y.cuda(), 5, yb.cuda(), cu.cuda(), seq_slot.cuda(), 3, max(lens),
+                               torch.float32)
             _near(got, want, 1e-4); _near(s_got, s_want, 1e-4)
