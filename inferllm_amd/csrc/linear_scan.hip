@@ -290,50 +290,70 @@ extern "C" int illm_gla_prepare(const void* U, int dt, int u_stride, int q_off, 
 // lru_gates gives a and x; lru_scan runs the recurrence from the kept state [slots][C] and back
 // into it and multiplies by the other branch.  All float32 but the stored Y and the output.
 //
-// grid (ceil(T / LRU_ROWS), nb); 256 threads over a block's outputs; the rows' inputs go through
-// LDS.  Wt [2][nb][cb in][cb out] float32: the two maps transposed, so that the threads of a wave
-// read neighbouring outputs of one input.
-#define LRU_ROWS 16
+// grid (ceil(T / ROWS), nb); 256 threads over a block's outputs; the rows' inputs go through LDS, laid
+// out [input][row] so that a thread reads one input of all its rows in 16-byte pieces.  Steps of few
+// rows take tiles of 4 rows (more blocks), longer ones tiles of 16.  Wt [2][nb][cb in][cb out] float32:
+// the two maps transposed, so that the threads of a wave read neighbouring outputs of one input.
+template <int ROWS>
 __global__ void __launch_bounds__(256)
 lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, const float* __restrict__ br,
                  const float* __restrict__ bi, const float* __restrict__ lam, float rate,
                  float* __restrict__ a_out, float* __restrict__ x_out, int T, int C, int cb) {
-    extern __shared__ float us[];                   // [LRU_ROWS][cb]
-    const int t0 = blockIdx.x * LRU_ROWS, b = blockIdx.y, nb = C / cb;
-    const int rows = min(LRU_ROWS, T - t0);
-    for (int e = threadIdx.x; e < LRU_ROWS * cb; e += 256) {
+    extern __shared__ float us[];                   // [cb][ROWS]
+    const int t0 = blockIdx.x * ROWS, b = blockIdx.y, nb = C / cb;
+    const int rows = min(ROWS, T - t0);
+    for (int e = threadIdx.x; e < ROWS * cb; e += 256) {
         const int r = e / cb, i = e - r * cb;
-        us[e] = r < rows ? u[(size_t)(t0 + r) * C + (size_t)b * cb + i] : 0.f;
+        us[i * ROWS + r] = r < rows ? u[(size_t)(t0 + r) * C + (size_t)b * cb + i] : 0.f;
     }
     __syncthreads();
     const float* wr = Wt + (size_t)b * cb * cb;
     const float* wi = Wt + ((size_t)nb + b) * cb * cb;
     for (int o = threadIdx.x; o < cb; o += 256) {
-        float ar[LRU_ROWS], ai[LRU_ROWS];
+        float ar[ROWS], ai[ROWS];
 #pragma unroll
-        for (int r = 0; r < LRU_ROWS; ++r) ar[r] = ai[r] = 0.f;
-#pragma unroll 8
+        for (int r = 0; r < ROWS; ++r) ar[r] = ai[r] = 0.f;
+#pragma unroll 4
         for (int i = 0; i < cb; ++i) {
             const float w1 = wr[(size_t)i * cb + o], w2 = wi[(size_t)i * cb + o];
+            const float4* xr = (const float4*)(us + i * ROWS);
 #pragma unroll
-            for (int r = 0; r < LRU_ROWS; ++r) {
-                const float x = us[r * cb + i];
-                ar[r] = fmaf(w1, x, ar[r]);
-                ai[r] = fmaf(w2, x, ai[r]);
+            for (int r4 = 0; r4 < ROWS / 4; ++r4) {
+                const float4 x = xr[r4];
+                ar[4 * r4 + 0] = fmaf(w1, x.x, ar[4 * r4 + 0]); ai[4 * r4 + 0] = fmaf(w2, x.x, ai[4 * r4 + 0]);
+                ar[4 * r4 + 1] = fmaf(w1, x.y, ar[4 * r4 + 1]); ai[4 * r4 + 1] = fmaf(w2, x.y, ai[4 * r4 + 1]);
+                ar[4 * r4 + 2] = fmaf(w1, x.z, ar[4 * r4 + 2]); ai[4 * r4 + 2] = fmaf(w2, x.z, ai[4 * r4 + 2]);
+                ar[4 * r4 + 3] = fmaf(w1, x.w, ar[4 * r4 + 3]); ai[4 * r4 + 3] = fmaf(w2, x.w, ai[4 * r4 + 3]);
             }
         }
         const int c = b * cb + o;
         const float sp = ls_softplus(lam[c]), b1 = br[c], b2 = bi[c];
 #pragma unroll
-        for (int r = 0; r < LRU_ROWS; ++r) {
+        for (int r = 0; r < ROWS; ++r) {
             if (r >= rows) continue;
             const float rg = ls_sigmoid(ar[r] + b1), ig = ls_sigmoid(ai[r] + b2);
             const float log_a = -rate * rg * sp;
             a_out[(size_t)(t0 + r) * C + c] = expf(log_a);
             // 1 - a^2 as -expm1(2 log a): a decay close to 1 keeps its digits
-            x_out[(size_t)(t0 + r) * C + c] = sqrtf(fmaxf(-expm1f(2.0f * log_a), 0.f)) * ig * us[r * cb + o];
+            x_out[(size_t)(t0 + r) * C + c] = sqrtf(fmaxf(-expm1f(2.0f * log_a), 0.f)) * ig * us[o * ROWS + r];
         }
     }
+}
+
+template <int ROWS>
+static int lru_gates_launch(const float* u, const float* Wt, const float* br, const float* bi,
+                            const float* lam, float rate, float* a_out, float* x_out, int T, int C,
+                            int nb, hipStream_t st) {
+    const int cb = C / nb;
+    const size_t lds = (size_t)ROWS * cb * sizeof(float);
+    if (lds > 64 * 1024) return ILLM_ERR_ARG;
+    if (lds > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)lru_gates_kernel<ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+        return ILLM_ERR_LAUNCH;
+    hipLaunchKernelGGL(lru_gates_kernel<ROWS>, dim3((T + ROWS - 1) / ROWS, nb), dim3(256), lds, st, u, Wt, br,
+                       bi, lam, rate, a_out, x_out, T, C, cb);
+    return illm_launch_status();
 }
 
 extern "C" int illm_lru_gates(const float* u, const float* Wt, const float* br, const float* bi,
@@ -341,16 +361,8 @@ extern "C" int illm_lru_gates(const float* u, const float* Wt, const float* br, 
                               int nb, void* stream) {
     if (T < 0 || C <= 0 || nb <= 0 || C % nb || nb > 65535) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    const int cb = C / nb;
-    const size_t lds = (size_t)LRU_ROWS * cb * sizeof(float);
-    if (lds > 64 * 1024) return ILLM_ERR_ARG;
-    if (lds > 48 * 1024 &&
-        hipFuncSetAttribute((const void*)lru_gates_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess)
-        return ILLM_ERR_LAUNCH;
-    hipLaunchKernelGGL(lru_gates_kernel, dim3((T + LRU_ROWS - 1) / LRU_ROWS, nb), dim3(256), lds,
-                       (hipStream_t)stream, u, Wt, br, bi, lam, rate, a_out, x_out, T, C, cb);
-    return illm_launch_status();
+    if (T <= 128) return lru_gates_launch<4>(u, Wt, br, bi, lam, rate, a_out, x_out, T, C, nb, (hipStream_t)stream);
+    return lru_gates_launch<16>(u, Wt, br, bi, lam, rate, a_out, x_out, T, C, nb, (hipStream_t)stream);
 }
 
 __device__ __forceinline__ float ls_gelu_tanh(float z) {
