@@ -299,7 +299,7 @@ __global__ void __launch_bounds__(256)
 lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, const float* __restrict__ br,
                  const float* __restrict__ bi, const float* __restrict__ lam, float rate,
                  float* __restrict__ a_out, float* __restrict__ x_out, int T, int C, int cb) {
-    extern __shared__ float us[];                   // [cb][ROWS]
+    extern __shared__ float us[];                   // [cb][ROWS], then the slices' partial sums
     const int t0 = blockIdx.x * ROWS, b = blockIdx.y, nb = C / cb;
     const int rows = min(ROWS, T - t0);
     for (int e = threadIdx.x; e < ROWS * cb; e += 256) {
@@ -309,23 +309,54 @@ lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ Wt, cons
     __syncthreads();
     const float* wr = Wt + (size_t)b * cb * cb;
     const float* wi = Wt + ((size_t)nb + b) * cb * cb;
-    for (int o = threadIdx.x; o < cb; o += 256) {
+    // a block narrower than the thread block cuts its inputs into S slices, one a group of cb
+    // threads, whose sums are added in slice order
+    const int S = cb < 256 ? 256 / cb : 1;
+    const int per = (cb + S - 1) / S;
+    float* part = us + (size_t)cb * ROWS;           // [S][cb][2 ROWS]
+    for (int o0 = 0; o0 < cb; o0 += 256) {
+        const int o = S > 1 ? (int)threadIdx.x % cb : o0 + (int)threadIdx.x;
+        const int sl = S > 1 ? (int)threadIdx.x / cb : 0;
+        const bool live = o < cb && sl < S;
         float ar[ROWS], ai[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) ar[r] = ai[r] = 0.f;
-#pragma unroll 4
-        for (int i = 0; i < cb; ++i) {
-            const float w1 = wr[(size_t)i * cb + o], w2 = wi[(size_t)i * cb + o];
-            const float4* xr = (const float4*)(us + i * ROWS);
+        if (live) {
+            const int i_lo = sl * per, i_hi = min(cb, i_lo + per);
+#pragma unroll 8
+            for (int i = i_lo; i < i_hi; ++i) {
+                const float w1 = wr[(size_t)i * cb + o], w2 = wi[(size_t)i * cb + o];
+                const float4* xr = (const float4*)(us + i * ROWS);
 #pragma unroll
-            for (int r4 = 0; r4 < ROWS / 4; ++r4) {
-                const float4 x = xr[r4];
-                ar[4 * r4 + 0] = fmaf(w1, x.x, ar[4 * r4 + 0]); ai[4 * r4 + 0] = fmaf(w2, x.x, ai[4 * r4 + 0]);
-                ar[4 * r4 + 1] = fmaf(w1, x.y, ar[4 * r4 + 1]); ai[4 * r4 + 1] = fmaf(w2, x.y, ai[4 * r4 + 1]);
-                ar[4 * r4 + 2] = fmaf(w1, x.z, ar[4 * r4 + 2]); ai[4 * r4 + 2] = fmaf(w2, x.z, ai[4 * r4 + 2]);
-                ar[4 * r4 + 3] = fmaf(w1, x.w, ar[4 * r4 + 3]); ai[4 * r4 + 3] = fmaf(w2, x.w, ai[4 * r4 + 3]);
+                for (int r4 = 0; r4 < ROWS / 4; ++r4) {
+                    const float4 x = xr[r4];
+                    ar[4 * r4 + 0] = fmaf(w1, x.x, ar[4 * r4 + 0]); ai[4 * r4 + 0] = fmaf(w2, x.x, ai[4 * r4 + 0]);
+                    ar[4 * r4 + 1] = fmaf(w1, x.y, ar[4 * r4 + 1]); ai[4 * r4 + 1] = fmaf(w2, x.y, ai[4 * r4 + 1]);
+                    ar[4 * r4 + 2] = fmaf(w1, x.z, ar[4 * r4 + 2]); ai[4 * r4 + 2] = fmaf(w2, x.z, ai[4 * r4 + 2]);
+                    ar[4 * r4 + 3] = fmaf(w1, x.w, ar[4 * r4 + 3]); ai[4 * r4 + 3] = fmaf(w2, x.w, ai[4 * r4 + 3]);
+                }
             }
         }
+        if (S > 1) {
+            if (live) {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    part[((size_t)sl * cb + o) * 2 * ROWS + r] = ar[r];
+                    part[((size_t)sl * cb + o) * 2 * ROWS + ROWS + r] = ai[r];
+                }
+            }
+            __syncthreads();
+            if (live && sl == 0) {
+                for (int s2 = 1; s2 < S; ++s2) {
+#pragma unroll
+                    for (int r = 0; r < ROWS; ++r) {
+                        ar[r] += part[((size_t)s2 * cb + o) * 2 * ROWS + r];
+                        ai[r] += part[((size_t)s2 * cb + o) * 2 * ROWS + ROWS + r];
+                    }
+                }
+            }
+        }
+        if (!live || sl != 0) continue;
         const int c = b * cb + o;
         const float sp = ls_softplus(lam[c]), b1 = br[c], b2 = bi[c];
 #pragma unroll
@@ -345,7 +376,8 @@ static int lru_gates_launch(const float* u, const float* Wt, const float* br, co
                             const float* lam, float rate, float* a_out, float* x_out, int T, int C,
                             int nb, hipStream_t st) {
     const int cb = C / nb;
-    const size_t lds = (size_t)ROWS * cb * sizeof(float);
+    const int slices = cb < 256 ? 256 / cb : 1;
+    const size_t lds = ((size_t)ROWS * cb + (slices > 1 ? (size_t)slices * cb * 2 * ROWS : 0)) * sizeof(float);
     if (lds > 64 * 1024) return ILLM_ERR_ARG;
     if (lds > 48 * 1024 &&
         hipFuncSetAttribute((const void*)lru_gates_kernel<ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -30,8 +30,13 @@ short_conv_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
     const int r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c >= C) return;
     const int K = taps - 1, slot = row_slot[r];
+    int above[CONV_MAX_TAPS];                   // the slots of the rows above, all asked for at once
+#pragma unroll
+    for (int j = 1; j < CONV_MAX_TAPS; ++j) above[j] = (j <= K && r - j >= 0) ? row_slot[r - j] : -1;
     int n = 0;                                  // rows of the same sequence right above this one
-    while (n < K && r - n - 1 >= 0 && row_slot[r - n - 1] == slot) ++n;
+#pragma unroll
+    for (int j = 1; j < CONV_MAX_TAPS; ++j)
+        if (n == j - 1 && above[j] == slot) n = j;
     const float ib = in_bias ? in_bias[c] : 0.f;
     float in[CONV_MAX_TAPS];                    // in[j]: the input taps - 1 - j rows back
 #pragma unroll
@@ -152,9 +157,39 @@ clamped_swish_mul_kernel(const void* __restrict__ gu, void* __restrict__ out, in
     st_f(out, dt, t * F + f, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
 }
 
+// bfloat16 rows with F % 8 == 0: 8 values (16 bytes) of gate and of up a thread
+__global__ void __launch_bounds__(256)
+clamped_swish_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int F, float limit,
+                                float alpha) {
+    const size_t t = blockIdx.y;
+    const int f = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (f >= F) return;
+    const uint4 g = *(const uint4*)(gu + t * 2 * F + f);
+    const uint4 u = *(const uint4*)(gu + t * 2 * F + F + f);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float g0 = fminf(__uint_as_float(gw[i] << 16), limit), g1 = fminf(__uint_as_float(gw[i] & 0xffff0000u), limit);
+        const float u0 = fminf(fmaxf(__uint_as_float(uw[i] << 16), -limit), limit);
+        const float u1 = fminf(fmaxf(__uint_as_float(uw[i] & 0xffff0000u), -limit), limit);
+        ow[i] = pack_bf16x2(g0 / (1.0f + expf(-alpha * g0)) * (u0 + 1.0f), g1 / (1.0f + expf(-alpha * g1)) * (u1 + 1.0f));
+    }
+    *(uint4*)(out + t * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, int T, int F,
                                       float limit, float alpha, void* stream) {
     if (T < 0 || F <= 0 || !illm_dtype_ok(dt) || !(limit > 0.f)) return ILLM_ERR_ARG;
+    if (dt == ILLM_BF16 && F % 8 == 0) {
+        for (int t0 = 0; t0 < T; t0 += 65535) {
+            const int rows = T - t0 < 65535 ? T - t0 : 65535;
+            hipLaunchKernelGGL(clamped_swish_mul_bf16x8_kernel, dim3((F / 8 + 255) / 256, rows), dim3(256), 0,
+                               (hipStream_t)stream, (const bf16_t*)gate_up + (size_t)t0 * 2 * F,
+                               (bf16_t*)out + (size_t)t0 * F, F, limit, alpha);
+        }
+        return illm_launch_status();
+    }
     const size_t esz = dt == ILLM_BF16 ? 2 : 4;
     for (int t0 = 0; t0 < T; t0 += 65535) {
         const int rows = T - t0 < 65535 ? T - t0 : 65535;
@@ -212,12 +247,15 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
     const int slot = conv_w ? row_slot[r] : 0;
     if (NV > 0) {
         const int n4 = E / 4;
-        float4 xv[NV > 0 ? NV : 1], av[NV > 0 ? NV : 1];
+        float4 xv[NV > 0 ? NV : 1], av[NV > 0 ? NV : 1], pwv[NV > 0 ? NV : 1], wv4[NV > 0 ? NV : 1];
+        const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const int i4 = threadIdx.x + 256 * k;
-            xv[k] = i4 < n4 ? ((const float4*)(x + ib))[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
-            av[k] = (a && i4 < n4) ? sc_ld4(a, a_dt, ib / 4 + i4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            xv[k] = i4 < n4 ? ((const float4*)(x + ib))[i4] : zero4;
+            av[k] = (a && i4 < n4) ? sc_ld4(a, a_dt, ib / 4 + i4) : zero4;
+            pwv[k] = (a && i4 < n4) ? sc_ld4(post_w, post_w_dt, i4) : zero4;
+            wv4[k] = i4 < n4 ? sc_ld4(w, w_dt, i4) : zero4;
         }
         if (a) {
             float sa = 0.f;
@@ -229,7 +267,7 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
             for (int k = 0; k < NV; ++k) {
                 const int i4 = threadIdx.x + 256 * k;
                 if (i4 >= n4) continue;
-                const float4 pw = sc_ld4(post_w, post_w_dt, i4);
+                const float4 pw = pwv[k];
                 xv[k].x += gain * (av[k].x * inv_a * pw.x);
                 xv[k].y += gain * (av[k].y * inv_a * pw.y);
                 xv[k].z += gain * (av[k].z * inv_a * pw.z);
@@ -246,7 +284,7 @@ post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a
         for (int k = 0; k < NV; ++k) {
             const int i4 = threadIdx.x + 256 * k;
             if (i4 >= n4) continue;
-            const float4 wv = sc_ld4(w, w_dt, i4);
+            const float4 wv = wv4[k];
             float h[4] = {(xv[k].x * scale) * wv.x, (xv[k].y * scale) * wv.y, (xv[k].z * scale) * wv.z,
                           (xv[k].w * scale) * wv.w};
             if (conv_w) {
