@@ -20,6 +20,82 @@ __device__ __forceinline__ float conv_round(float v, int dt) {
     return dt == ILLM_BF16 ? bf16_to_f32(f32_to_bf16(v)) : v;
 }
 
+__device__ __forceinline__ float4 sc_ld4(const void* p, int dt, size_t i4) {
+    if (dt == ILLM_BF16) {
+        const uint2 u = ((const uint2*)p)[i4];
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+    }
+    return ((const float4*)p)[i4];
+}
+
+__device__ __forceinline__ void sc_st4(void* p, int dt, size_t i4, float4 v) {
+    if (dt == ILLM_BF16) {
+        uint2 u;
+        u.x = pack_bf16x2(v.x, v.y);
+        u.y = pack_bf16x2(v.z, v.w);
+        ((uint2*)p)[i4] = u;
+    } else {
+        ((float4*)p)[i4] = v;
+    }
+}
+
+// Four channels a thread where the rows allow (C, the offset and the strides multiples of 4): grid
+// (rows, ceil(C / 1024)).
+__global__ void __launch_bounds__(256)
+short_conv_vec4_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
+                       const float* __restrict__ in_bias, const float* __restrict__ w,
+                       const float* __restrict__ bias, int taps, void* __restrict__ tail, int tail_dt,
+                       const int32_t* __restrict__ row_slot, int add_input, void* __restrict__ out,
+                       int out_dt, int out_stride, int C, int update_tail) {
+    const int r = blockIdx.x, c4 = blockIdx.y * 256 + threadIdx.x;
+    if (4 * c4 >= C) return;
+    const int K = taps - 1, slot = row_slot[r];
+    int above[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 1; j < CONV_MAX_TAPS; ++j) above[j] = (j <= K && r - j >= 0) ? row_slot[r - j] : -1;
+    int n = 0;
+#pragma unroll
+    for (int j = 1; j < CONV_MAX_TAPS; ++j)
+        if (n == j - 1 && above[j] == slot) n = j;
+    float4 ib = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (in_bias) ib = ((const float4*)in_bias)[c4];
+    float4 in[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) continue;
+        const int back = K - j;
+        if (back <= n) {
+            float4 v = sc_ld4(X, x_dt, ((size_t)(r - back) * x_stride + x_off) / 4 + c4);
+            v.x += ib.x; v.y += ib.y; v.z += ib.z; v.w += ib.w;
+            if (in_bias) {
+                v.x = conv_round(v.x, tail_dt); v.y = conv_round(v.y, tail_dt);
+                v.z = conv_round(v.z, tail_dt); v.w = conv_round(v.w, tail_dt);
+            }
+            in[j] = v;
+        } else {
+            in[j] = sc_ld4(tail, tail_dt, ((size_t)slot * K + (K - (back - n))) * (C / 4) + c4);
+        }
+    }
+    float y[4];
+    if (bias) { const float4 b4 = ((const float4*)bias)[c4]; y[0] = b4.x; y[1] = b4.y; y[2] = b4.z; y[3] = b4.w; }
+    else y[0] = y[1] = y[2] = y[3] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float* cw = w + (size_t)(4 * c4 + e) * taps;
+#pragma unroll
+        for (int j = 0; j < CONV_MAX_TAPS; ++j)
+            if (j < taps) y[e] = fmaf(cw[j], ((const float*)&in[j])[e], y[e]);
+        if (add_input) y[e] += ((const float*)&in[K])[e];
+    }
+    sc_st4(out, out_dt, ((size_t)r * out_stride) / 4 + c4, make_float4(y[0], y[1], y[2], y[3]));
+    if (update_tail) {
+#pragma unroll
+        for (int j = 1; j < CONV_MAX_TAPS; ++j)
+            if (j < taps) sc_st4(tail, tail_dt, ((size_t)slot * K + (j - 1)) * (C / 4) + c4, in[j]);
+    }
+}
+
 // grid (rows, ceil(C / 256)); 256 threads, one a channel.
 __global__ void __launch_bounds__(256)
 short_conv_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
@@ -72,6 +148,12 @@ extern "C" int illm_short_conv(const void* X, int x_dt, int x_stride, int x_off,
         out_stride < C || (C + 255) / 256 > 65535)
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
+    if (C % 4 == 0 && x_off % 4 == 0 && x_stride % 4 == 0 && out_stride % 4 == 0) {
+        hipLaunchKernelGGL(short_conv_vec4_kernel, dim3(T, (C / 4 + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                           X, x_dt, x_stride, x_off, in_bias, w, bias, taps, tail, tail_dt, row_slot,
+                           add_input, out, out_dt, out_stride, C, taps > 1 ? update_tail : 0);
+        return illm_launch_status();
+    }
     hipLaunchKernelGGL(short_conv_kernel, dim3(T, (C + 255) / 256), dim3(256), 0, (hipStream_t)stream,
                        X, x_dt, x_stride, x_off, in_bias, w, bias, taps, tail, tail_dt, row_slot,
                        add_input, out, out_dt, out_stride, C, taps > 1 ? update_tail : 0);
@@ -210,26 +292,6 @@ extern "C" int illm_clamped_swish_mul(const void* gate_up, void* out, int dt, in
 // grid (rows); 256 threads.  A thread owns NV groups of 4 consecutive columns (E % 4 == 0, E <= 1024
 // NV) and asks for everything it reads of a pass before it uses any of it; other widths take the
 // plain loop (NV 0), which keeps the row's sum in LDS (E floats) between the passes.
-__device__ __forceinline__ float4 sc_ld4(const void* p, int dt, size_t i4) {
-    if (dt == ILLM_BF16) {
-        const uint2 u = ((const uint2*)p)[i4];
-        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
-                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
-    }
-    return ((const float4*)p)[i4];
-}
-
-__device__ __forceinline__ void sc_st4(void* p, int dt, size_t i4, float4 v) {
-    if (dt == ILLM_BF16) {
-        uint2 u;
-        u.x = pack_bf16x2(v.x, v.y);
-        u.y = pack_bf16x2(v.z, v.w);
-        ((uint2*)p)[i4] = u;
-    } else {
-        ((float4*)p)[i4] = v;
-    }
-}
-
 template <int NV>
 __global__ void __launch_bounds__(256)
 post_add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ a, int a_dt,

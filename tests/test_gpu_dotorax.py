@@ -440,10 +440,11 @@ def test_short_convolution_with_a_kept_tail_against_plain_torch(lens, dtype):
     from inferllm_amd.kernels import ops
     g = torch.Generator().manual_seed(sum(lens))
     tol = 1e-5 if dtype == torch.float32 else 2e-2
-    for C, taps, off in ((70, 4, 5), (300, 2, 0), (9, 1, 3), (33, 8, 0)):
+    for C, taps, off in ((70, 4, 5), (300, 2, 0), (9, 1, 3), (33, 8, 0), (64, 3, 4), (1028, 4, 8)):
         T = sum(lens)
         cu, seq_slot, row_slot = _packed(lens, [4, 0, 2][:len(lens)])
-        X = torch.randn(T, C + off + 2, generator=g).to(dtype)
+        # (rows whose width, offset and channels are multiples of 4 take four channels a thread)
+        X = torch.randn(T, C + off + (2 if C % 4 else 4), generator=g).to(dtype)
         w, bias, in_bias = torch.randn(C, taps, generator=g), torch.randn(C, generator=g), torch.randn(C, generator=g)
         tail = torch.randn(6, max(taps - 1, 1), C, generator=g).to(dtype)
         single = max(lens) == 1
