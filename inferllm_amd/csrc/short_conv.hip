@@ -60,7 +60,8 @@ short_conv_vec4_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x
         if (n == j - 1 && above[j] == slot) n = j;
     float4 ib = make_float4(0.f, 0.f, 0.f, 0.f);
     if (in_bias) ib = ((const float4*)in_bias)[c4];
-    float4 in[CONV_MAX_TAPS];
+    float4 in[CONV_MAX_TAPS];                   // (indexed by constants only: the array stays in registers)
+    float4 cur = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
         if (j >= taps) continue;
@@ -76,6 +77,7 @@ short_conv_vec4_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x
         } else {
             in[j] = sc_ld4(tail, tail_dt, ((size_t)slot * K + (K - (back - n))) * (C / 4) + c4);
         }
+        if (back == 0) cur = in[j];
     }
     float y[4];
     if (bias) { const float4 b4 = ((const float4*)bias)[c4]; y[0] = b4.x; y[1] = b4.y; y[2] = b4.z; y[3] = b4.w; }
@@ -86,7 +88,7 @@ short_conv_vec4_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x
 #pragma unroll
         for (int j = 0; j < CONV_MAX_TAPS; ++j)
             if (j < taps) y[e] = fmaf(cw[j], ((const float*)&in[j])[e], y[e]);
-        if (add_input) y[e] += ((const float*)&in[K])[e];
+        if (add_input) y[e] += ((const float*)&cur)[e];
     }
     sc_st4(out, out_dt, ((size_t)r * out_stride) / 4 + c4, make_float4(y[0], y[1], y[2], y[3]));
     if (update_tail) {
@@ -114,7 +116,8 @@ short_conv_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
     for (int j = 1; j < CONV_MAX_TAPS; ++j)
         if (n == j - 1 && above[j] == slot) n = j;
     const float ib = in_bias ? in_bias[c] : 0.f;
-    float in[CONV_MAX_TAPS];                    // in[j]: the input taps - 1 - j rows back
+    float in[CONV_MAX_TAPS];                    // in[j]: the input taps - 1 - j rows back (indexed by
+    float cur = 0.f;                            // constants only: the array stays in registers)
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
         if (j >= taps) continue;
@@ -125,12 +128,13 @@ short_conv_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x_off,
         } else {
             in[j] = ld_f(tail, tail_dt, ((size_t)slot * K + (K - (back - n))) * C + c);
         }
+        if (back == 0) cur = in[j];
     }
     float y = bias ? bias[c] : 0.f;
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j)
         if (j < taps) y = fmaf(w[(size_t)c * taps + j], in[j], y);
-    if (add_input) y += in[K];
+    if (add_input) y += cur;
     st_f(out, out_dt, (size_t)r * out_stride + c, y);
     if (update_tail) {
 #pragma unroll
