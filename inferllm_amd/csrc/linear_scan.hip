@@ -393,7 +393,9 @@ extern "C" int illm_lru_gates(const float* u, const float* Wt, const float* br, 
                               int nb, void* stream) {
     if (T < 0 || C <= 0 || nb <= 0 || C % nb || nb > 65535) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    if (T <= 128) return lru_gates_launch<4>(u, Wt, br, bi, lam, rate, a_out, x_out, T, C, nb, (hipStream_t)stream);
+    // tiles of 16 rows where a block's inputs of 16 rows fit LDS (blocks of up to 1,024 channels)
+    if (T <= 128 || C / nb > 1024)
+        return lru_gates_launch<4>(u, Wt, br, bi, lam, rate, a_out, x_out, T, C, nb, (hipStream_t)stream);
     return lru_gates_launch<16>(u, Wt, br, bi, lam, rate, a_out, x_out, T, C, nb, (hipStream_t)stream);
 }
 

@@ -263,8 +263,8 @@ class GatedLinearRecurrence(Mixer):
             raise ValueError(f"gated linear recurrence: {channels} channels do not split into {blocks} equal blocks")
         if not 1 <= int(conv) <= 8:
             raise ValueError(f"gated linear recurrence: {conv} taps; the kernels take 1 to 8")
-        if int(channels) // int(blocks) > 1024:
-            raise ValueError("gated linear recurrence: blocks of more than 1024 channels are beyond the gates' kernel")
+        if int(channels) // int(blocks) > 4096:
+            raise ValueError("gated linear recurrence: blocks of more than 4096 channels are beyond the gates' kernel")
         self.E, self.C, self.nb, self.taps = int(hidden_size), int(channels), int(blocks), int(conv)
 
     def shapes(self) -> Dict[str, TensorWant]:

@@ -621,7 +621,7 @@ def test_linear_attention_and_recurrent_unit_kernels_against_plain_torch(dtype):
             got = ops.gla_prepare(U.cuda(), 0, H * dk + 3, 2 * H * dk + 4, Z.cuda(), zb.cuda(), 7.0, H, dk, dv)
             for a, b in zip(got, want):
                 _near(a, b, 1e-5)
-        for C, nb in ((24, 3), (300, 1), (64, 8)):
+        for C, nb in ((24, 3), (300, 1), (64, 8), (1100, 1)):
             cb = C // nb
             u = torch.randn(T, C, generator=g) * 2
             wt = torch.randn(2, nb, cb, cb, generator=g) * 0.5
