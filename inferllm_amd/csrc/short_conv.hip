@@ -54,20 +54,29 @@ short_conv_vec4_kernel(const void* __restrict__ X, int x_dt, int x_stride, int x
     int above[CONV_MAX_TAPS];
 #pragma unroll
     for (int j = 1; j < CONV_MAX_TAPS; ++j) above[j] = (j <= K && r - j >= 0) ? row_slot[r - j] : -1;
+    float4 ib = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (in_bias) ib = ((const float4*)in_bias)[c4];
+    // the rows above are asked for together with their slots, before it is known how many of them
+    // belong to this sequence (a row of another sequence is then read and dropped): one trip to
+    // memory instead of two in a row
+    float4 in[CONV_MAX_TAPS];                   // (indexed by constants only: the array stays in registers)
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) continue;
+        const int rr = max(r - (K - j), 0);
+        in[j] = sc_ld4(X, x_dt, ((size_t)rr * x_stride + x_off) / 4 + c4);
+    }
     int n = 0;
 #pragma unroll
     for (int j = 1; j < CONV_MAX_TAPS; ++j)
         if (n == j - 1 && above[j] == slot) n = j;
-    float4 ib = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (in_bias) ib = ((const float4*)in_bias)[c4];
-    float4 in[CONV_MAX_TAPS];                   // (indexed by constants only: the array stays in registers)
     float4 cur = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
         if (j >= taps) continue;
         const int back = K - j;
         if (back <= n) {
-            float4 v = sc_ld4(X, x_dt, ((size_t)(r - back) * x_stride + x_off) / 4 + c4);
+            float4 v = in[j];
             v.x += ib.x; v.y += ib.y; v.z += ib.z; v.w += ib.w;
             if (in_bias) {
                 v.x = conv_round(v.x, tail_dt); v.y = conv_round(v.y, tail_dt);
