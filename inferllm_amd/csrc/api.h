@@ -216,6 +216,11 @@ int illm_gemm_rows_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M,
                         const float* ssq, int parts, float eps, void* stream);
 int illm_gemm_rows_gateup_silu(const void* X, const void* Wt, void* Y, int y_dt, int M, int F,
                                int K, const float* ssq, int parts, float eps, void* stream);
+// The same with the clamped gate in place of SiLU where limit > 0: Y = g sigmoid(alpha g) (u + 1),
+// g = min(gate, limit), u = clamp(up, -limit, limit) (limit 0: SiLU as above).
+int illm_gemm_rows_gateup_act(const void* X, const void* Wt, void* Y, int y_dt, int M, int F, int K,
+                              const float* ssq, int parts, float eps, float limit, float alpha,
+                              void* stream);
 int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int K,
                              const float* cos_sin, int max_pos, const int32_t* row_pos,
                              const int32_t* row_slot, void* kcache, void* vcache,
@@ -228,6 +233,10 @@ int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int 
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y, int y_dt,
                                  int M, int F, int K, const float* ssq, int parts, float eps,
                                  int waves_wanted, void* stream);
+// The same with the clamped gate where limit > 0 (as illm_gemm_rows_gateup_act).
+int illm_gemm_skinny_gateup_act(const void* X, const void* W, const void* Wt, void* Y, int y_dt,
+                                int M, int F, int K, const float* ssq, int parts, float eps,
+                                int waves_wanted, float limit, float alpha, void* stream);
 
 // Few bfloat16 rows (M <= 16, hd % 16 == 0): the q|k|v product, the rotation of q and k (pairs
 // (i, i + hd/2), all dims) at row_pos[m], q into Y[M, (nh + 2 nkv) hd] (k and v parts untouched),

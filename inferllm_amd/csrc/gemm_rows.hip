@@ -53,6 +53,8 @@ struct GrScale {
     const float* ssq;
     int parts;
     float eps;
+    float act_limit;             // gate|up: > 0, the clamped gate g sigmoid(act_alpha g) (u + 1) with
+    float act_alpha;             // g = min(gate, limit), u = clamp(up, -limit, limit); else silu(gate) up
 };
 
 // GR_PIECE: k-steps of 32 in a piece.  A block of four or more tiles has at most two parts of K,
@@ -279,7 +281,15 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
                 const int n0 = tile * 8 + q * 4;             // N is F here
                 float y[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) y[i] = (v[i] / (1.0f + expf(-v[i]))) * o[i];
+                for (int i = 0; i < 4; ++i) {
+                    if (scale.act_limit > 0.f) {
+                        const float gc = fminf(v[i], scale.act_limit);
+                        const float uc = fminf(fmaxf(o[i], -scale.act_limit), scale.act_limit);
+                        y[i] = gc / (1.0f + expf(-scale.act_alpha * gc)) * (uc + 1.0f);
+                    } else {
+                        y[i] = (v[i] / (1.0f + expf(-v[i]))) * o[i];
+                    }
+                }
                 const size_t at = (size_t)m * N + n0;
                 if (n0 + 3 < N && (N & 3) == 0 && y_dt == ILLM_BF16) {
                     *(uint2*)((bf16_t*)Y + at) =
@@ -434,13 +444,21 @@ extern "C" int illm_gemm_rows_bf16(const void* X, const void* Wt, void* Y, int y
                                   (hipStream_t)stream);
 }
 
+// With limit > 0 the clamped gate in place of SiLU: Y = g sigmoid(alpha g) (u + 1), g = min(gate, limit),
+// u = clamp(up, -limit, limit).
+extern "C" int illm_gemm_rows_gateup_act(const void* X, const void* Wt, void* Y, int y_dt, int M,
+                                         int F, int K, const float* ssq, int parts, float eps,
+                                         float limit, float alpha, void* stream) {
+    if (!rows_args_ok(X, Wt, Y, M, F, K, ssq, parts) || !illm_dtype_ok(y_dt) || limit < 0.f) return ILLM_ERR_ARG;
+    const GrScale scale = {ssq, parts, eps, limit, alpha};
+    return rows_product<GR_GATE_UP>(X, Wt, Y, y_dt, M, F, K, (F + 7) / 8, GrRope(), scale,
+                                    (hipStream_t)stream);
+}
+
 extern "C" int illm_gemm_rows_gateup_silu(const void* X, const void* Wt, void* Y, int y_dt, int M,
                                           int F, int K, const float* ssq, int parts, float eps,
                                           void* stream) {
-    if (!rows_args_ok(X, Wt, Y, M, F, K, ssq, parts) || !illm_dtype_ok(y_dt)) return ILLM_ERR_ARG;
-    const GrScale scale = {ssq, parts, eps};
-    return rows_product<GR_GATE_UP>(X, Wt, Y, y_dt, M, F, K, (F + 7) / 8, GrRope(), scale,
-                                    (hipStream_t)stream);
+    return illm_gemm_rows_gateup_act(X, Wt, Y, y_dt, M, F, K, ssq, parts, eps, 0.f, 0.f, stream);
 }
 
 extern "C" int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int K,

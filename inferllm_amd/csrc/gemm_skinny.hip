@@ -58,6 +58,8 @@ struct SkResidual {
     const float* ssq;            // consumer: [M, parts] or null
     int parts;
     float eps;
+    float act_limit;             // gate|up: > 0, the clamped gate g sigmoid(act_alpha g) (u + 1) with
+    float act_alpha;             // g = min(gate, limit), u = clamp(up, -limit, limit); else silu(gate) up
 };
 
 // TILED (NTB == 1, K % 32 == 0): W is a copy laid out for this kernel, [tile][k-step][16 rows][32 k]
@@ -365,8 +367,16 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 if (n0 + i < N) {
-                    const float gi = g[i] * rs;
-                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (gi / (1.0f + expf(-gi))) * (u[i] * rs));
+                    const float gi = g[i] * rs, ui = u[i] * rs;
+                    float yv;
+                    if (res.act_limit > 0.f) {
+                        const float gc = fminf(gi, res.act_limit);
+                        const float uc = fminf(fmaxf(ui, -res.act_limit), res.act_limit);
+                        yv = gc / (1.0f + expf(-res.act_alpha * gc)) * (uc + 1.0f);
+                    } else {
+                        yv = (gi / (1.0f + expf(-gi))) * ui;
+                    }
+                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, yv);
                 }
         }
         return;
@@ -440,7 +450,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     }
 }
 
-static const SkResidual SK_NO_RESIDUAL = {0, nullptr, ILLM_BF16, nullptr, nullptr, nullptr, 0, 0.f};
+static const SkResidual SK_NO_RESIDUAL = {0, nullptr, ILLM_BF16, nullptr, nullptr, nullptr, 0, 0.f, 0.f, 0.f};
 
 template <int MT, int NTB, int U, int MODE = SK_PLAIN, bool TILED = false, bool ONE_SHOT = false>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
@@ -567,14 +577,18 @@ extern "C" int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T) with W = [Wg (F rows) | Wu (F rows)], [2F, K]:
 // the gate and up products and the SiLU-multiply in one kernel (src/core/graph.cpp:57-79).
 // ssq: as for illm_gemm_skinny_bf16.
-extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y,
-                                            int y_dt, int M, int F, int K, const float* ssq,
-                                            int parts, float eps, int waves_wanted, void* stream) {
+// With limit > 0 the clamped gate in place of SiLU: Y = g sigmoid(alpha g) (u + 1), g = min(gate, limit),
+// u = clamp(up, -limit, limit).
+extern "C" int illm_gemm_skinny_gateup_act(const void* X, const void* W, const void* Wt, void* Y,
+                                           int y_dt, int M, int F, int K, const float* ssq,
+                                           int parts, float eps, int waves_wanted, float limit,
+                                           float alpha, void* stream) {
     if (M <= 0 || M > 64 || F <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt) ||
-        !scale_args_ok(ssq, parts, M))
+        !scale_args_ok(ssq, parts, M) || limit < 0.f)
         return ILLM_ERR_ARG;
     SkResidual res = SK_NO_RESIDUAL;
     res.ssq = ssq; res.parts = parts; res.eps = eps;
+    res.act_limit = limit; res.act_alpha = alpha;
     hipStream_t st = (hipStream_t)stream;
     const int mt = (M + 15) / 16;
     const int blocks = (F + 7) / 8;
@@ -602,10 +616,17 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const 
     }
     switch (mt) {
         case 1: return launch_skinny<1, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
-        case 2: return launch_skinny<2, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
-        case 3: return launch_skinny<3, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
-        default: return launch_skinny<4, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 2: return launch_skinny<2, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
+        case 3: return launch_skinny<3, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
+        default: return launch_skinny<4, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
     }
+}
+
+extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y,
+                                            int y_dt, int M, int F, int K, const float* ssq,
+                                            int parts, float eps, int waves_wanted, void* stream) {
+    return illm_gemm_skinny_gateup_act(X, W, Wt, Y, y_dt, M, F, K, ssq, parts, eps, waves_wanted, 0.f, 0.f,
+                                       stream);
 }
 
 // Decode step of an attention layer's input side in one kernel: Y = X . Wqkv^T, the q and k heads

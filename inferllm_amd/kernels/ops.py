@@ -1025,6 +1025,15 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
 
     Few bfloat16 rows: one fused MFMA kernel.  Otherwise the product and `silu_mul`.
     x may be `NormedRows`."""
+    return gate_up_act(x, w_gate_up, 0.0)
+
+
+def gate_up_act(x, w_gate_up, limit: float = 0.0) -> torch.Tensor:
+    """The gate and up products of w_gate_up = [Wg | Wu] ([2F, K]) and their activation: with `limit`
+    0 silu(gate) * up, with `limit` > 0 the clamped gate g sigmoid(1.702 g) (u + 1), g = min(gate,
+    limit), u = clamp(up, -limit, limit).  Few bfloat16 rows: one fused MFMA kernel (the activation
+    acts on the float32 sums).  Otherwise the product and `silu_mul` / `clamped_swish_mul`."""
+    limit = float(limit)
     if isinstance(x, NormedRows) and (w_gate_up.dtype != torch.bfloat16 or w_gate_up.shape[0] % 2):
         x = x.rows()
     M, K = x.shape
@@ -1034,24 +1043,27 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
         xt = xt.contiguous()
         _gpu(xt, w_gate_up.tiled)
         y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)
-        _check(_lib().illm_gemm_rows_gateup_silu(_p(xt), _p(w_gate_up.tiled), _p(y), _code(y), M,
-                                                 F2 // 2, K, ssq, parts, eps, _stream()),
-               "gate_up_silu (rows)")
+        _check(_lib().illm_gemm_rows_gateup_act(_p(xt), _p(w_gate_up.tiled), _p(y), _code(y), M,
+                                                F2 // 2, K, ssq, parts, eps, ctypes.c_float(limit),
+                                                ctypes.c_float(SWISH_ALPHA), _stream()),
+               "gate_up_act (rows)")
         return y
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
             and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
         xt, ssq, parts, eps = _operand(x)
         wp, wt = _w(w_gate_up, "gate_up")
         _gpu(xt, wp)
-        _need(wp.dim() == 2 and wp.shape[1] == K, "gate_up_silu: shapes")
+        _need(wp.dim() == 2 and wp.shape[1] == K, "gate_up_act: shapes")
         y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)
-        _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(wp), wt, _p(y), _code(y), M,
-                                                   F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
-                                                   _stream()), "gate_up_silu")
+        _check(_lib().illm_gemm_skinny_gateup_act(_p(xt), _p(wp), wt, _p(y), _code(y), M,
+                                                  F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
+                                                  ctypes.c_float(limit), ctypes.c_float(SWISH_ALPHA),
+                                                  _stream()), "gate_up_act")
         return y
     if isinstance(x, NormedRows):
         x = x.rows()
-    return silu_mul(linear(x, plain_weight(w_gate_up)))
+    both = linear(x, plain_weight(w_gate_up))
+    return clamped_swish_mul(both, limit) if limit > 0 else silu_mul(both)
 
 
 # ------------------------------------------------------------------ attention

@@ -107,7 +107,7 @@ class DenseActivation(FeedForward):
 class ClampedGated(FeedForward):
     """down(g sigmoid(1.702 g) (u + 1)) with g = min(gate h, limit) and u = clamp(up h, -limit, limit):
     the clamped activation of the routed experts as a dense feed-forward; gate and up are one
-    fused product."""
+    fused product, which in steps of few bfloat16 rows also applies the activation."""
 
     graph_safe_prompts = True
 
@@ -124,14 +124,14 @@ class ClampedGated(FeedForward):
 
     def load(self, tensors) -> None:
         self.w_gate_up = ops.decode_weight(_fuse([self._take(tensors, "gate"), self._take(tensors, "up")]),
-                                           "plain", self.decode_copies)
+                                           "gate_up", self.decode_copies)
         self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous(), "plain", self.decode_copies)
 
     def tunables(self):
-        return (("plain", self.w_down, {}),)
+        return (("gate_up", self.w_gate_up, {}), ("plain", self.w_down, {}))
 
     def forward(self, h, ctx: StepContext):
-        return ops.linear(ops.clamped_swish_mul(ops.linear(h, self.w_gate_up), self.limit), self.w_down)
+        return ops.linear(ops.gate_up_act(h, self.w_gate_up, self.limit), self.w_down)
 
 
 @register_part("feed_forward", "routed_experts")

@@ -107,6 +107,11 @@ def gate_up_silu(x, w_gate_up):
     return silu_mul(linear(x, w_gate_up))
 
 
+def gate_up_act(x, w_gate_up, limit=0.0):
+    both = linear(x, w_gate_up)
+    return clamped_swish_mul(both, limit) if limit > 0 else silu_mul(both)
+
+
 def gemm_generic(x, w, out_dtype):
     return linear(x, w, out_dtype)
 
@@ -890,7 +895,7 @@ def patch(monkeypatch):
                  "stream_mix_norm", "kv_store2", "attn_cap_rows", "attn_cap_decode", "delta_prepare",
                  "delta_conv_tail", "delta_scan", "delta_finish", "qkv_norm_mix_store", "ssm_prepare",
                  "ssm_finish", "memory_prepare", "memory_finish", "embed_pairs", "remember_last", "gelu_tanh",
-                 "short_conv", "short_conv_tail", "rms_rows_gain", "post_add_rmsnorm", "clamped_swish_mul", "qk_rotate_store",
+                 "short_conv", "short_conv_tail", "rms_rows_gain", "post_add_rmsnorm", "gate_up_act", "clamped_swish_mul", "qk_rotate_store",
                  "pool_store", "attn_pooled_rows", "attn_pooled_decode", "gla_prepare", "lru_gates", "lru_scan"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(ops.ScaledSum, "tensor", scaled_sum_tensor)

@@ -489,6 +489,32 @@ def test_norm_with_a_gain_and_clamped_gate_against_plain_torch(dtype):
                 _near(got, want, tol); _near(x_got, x_want, 1e-5); _near(t_got, t_want, tol)
 
 
+@pytest.mark.parametrize("M, F, K", [(1, 344, 256), (8, 1000, 136), (16, 33, 1000), (40, 320, 96), (64, 2816, 1024),
+                                     (100, 640, 512), (300, 96, 64)])
+def test_gate_and_up_with_the_clamped_gate_against_plain_torch(M, F, K):
+    """The gate|up product with the clamped gate: the fused kernels of few bfloat16 rows (from the
+    plain matrix and from the copy in the kernels' tile order) and the product followed by the
+    activation's own kernel, in bfloat16 and float32."""
+    from inferllm_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + F)
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(2 * F, K, generator=g) * (3.0 / K ** 0.5)
+    for dtype, tol in ((torch.bfloat16, 3e-2), (torch.float32, 2e-5)):
+        xd, wd = x.to(dtype), w.to(dtype)
+        both = xd.double() @ wd.double().T
+        gate, up = torch.clamp(both[:, :F], max=1.25), torch.clamp(both[:, F:], -1.25, 1.25)
+        want = gate * torch.sigmoid(1.702 * gate) * (up + 1)
+        ways = [wd.cuda()]
+        if dtype == torch.bfloat16:
+            ways.append(ops.decode_weight(wd.cuda(), "gate_up", True))
+        for wv in ways:
+            _near(ops.gate_up_act(xd.cuda(), wv, 1.25), want, tol)
+    # limit 0 is SiLU times up, as before
+    both = x.to(torch.bfloat16).double() @ w.to(torch.bfloat16).double().T
+    want = both[:, :F] * torch.sigmoid(both[:, :F]) * both[:, F:]
+    _near(ops.gate_up_act(x.to(torch.bfloat16).cuda(), w.to(torch.bfloat16).cuda()), want, 3e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_pooled_window_attention_against_plain_torch(dtype):
     """Rotation with either pairing, the norm a head and the store; the pooled rows of completed
